@@ -1,0 +1,290 @@
+// Mixture-of-experts feed-forward: grouped top-k router, device-side grouping
+// of tokens by expert, grouped expert GEMMs, weighted combine.
+//
+// moe_route_kernel (one wave per token): scores = softmax(z) over all router
+//   outputs; choice = score + correction; router outputs form `groups` equal
+//   groups of neighbours, a group ranks by its best choice score and only the
+//   `keep` best groups stay eligible (the others count as -inf); the `top`
+//   best eligible choices are taken; the weights are the plain scores.
+// moe_plan_kernel (one workgroup): (token, k) pairs bucketed by expert without
+//   a host round trip: offsets[E + 2], perm[P] (pair ids in expert order; the
+//   identity bucket E last), pos[P] (where each pair sits).
+// moe_grouped_gemm_kernel: C = A . W_e^T per expert segment, 64 x 64 tiles,
+//   f32 accumulation over K in ascending order for every output element (so a
+//   pair's result does not depend on which other pairs share its tile). Mode
+//   1 gathers A rows by token and applies the SwiGLU epilogue to the (gate,
+//   up) weight row pairs; mode 0 reads the sorted activation rows.
+// moe_combine_kernel: out[t] = sum_k weight * (expert output | the input
+//   itself for an identity expert), f32.
+#include "seqmix.h"
+
+#define MOE_MAX_E 1024
+
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, 64);
+    const int oi = __shfl_xor(i, o, 64);
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+  }
+}
+
+__global__ __launch_bounds__(64) void moe_route_kernel(
+    const float* __restrict__ z, const float* __restrict__ corr, int E, int G, int keep, int top,
+    int* __restrict__ idx, float* __restrict__ wt) {
+  __shared__ float sc[MOE_MAX_E], ch[MOE_MAX_E], gs[MOE_MAX_E];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const float* zr = z + (size_t)t * E;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) {
+    const float v = expf(zr[e] - mx);
+    sc[e] = v;
+    sum += v;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+  for (int e = lane; e < E; e += 64) {
+    const float s = sc[e] * inv;
+    sc[e] = s;
+    ch[e] = corr ? s + corr[e] : s;
+  }
+  __syncthreads();
+  if (G > 1 && keep < G) {
+    const int per = E / G;
+    for (int g = lane; g < G; g += 64) {
+      float b = -INFINITY;
+      for (int j = 0; j < per; ++j) b = fmaxf(b, ch[g * per + j]);
+      gs[g] = b;
+    }
+    __syncthreads();
+    // the `keep` best groups are marked with +inf, then the rest is masked
+    for (int k = 0; k < keep; ++k) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int g = lane; g < G; g += 64) {
+        const float v = gs[g];
+        if (v != INFINITY && (v > bv || bi == 0x7fffffff)) { bv = v; bi = g; }
+      }
+      wave_argmax(bv, bi);
+      if (lane == 0 && bi < G) gs[bi] = INFINITY;
+      __syncthreads();
+    }
+    for (int e = lane; e < E; e += 64)
+      if (gs[e / per] != INFINITY) ch[e] = -INFINITY;
+    __syncthreads();
+  }
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = ch[e];
+      if (v != INFINITY && (v > bv || bi == 0x7fffffff)) { bv = v; bi = e; }
+    }
+    wave_argmax(bv, bi);
+    bi = min(max(bi, 0), E - 1);
+    if (lane == 0) {
+      idx[(size_t)t * top + k] = bi;
+      wt[(size_t)t * top + k] = sc[bi];
+      ch[bi] = INFINITY;                      // taken
+    }
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_plan_kernel(const int* __restrict__ idx, int P, int E,
+                                                       int* __restrict__ plan) {
+  __shared__ int cnt[MOE_MAX_E + 2];
+  int* offsets = plan;                // [E + 2]
+  int* perm = plan + E + 2;           // [P]
+  int* pos = perm + P;                // [P]
+  for (int e = threadIdx.x; e < E + 2; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = min(max(idx[p], 0), E);     // identity experts share bucket E
+    atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e <= E; ++e) {
+      const int c = cnt[e];
+      offsets[e] = run;
+      cnt[e] = run;                           // becomes the fill cursor
+      run += c;
+    }
+    offsets[E + 1] = run;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = min(max(idx[p], 0), E);
+    const int s = atomicAdd(&cnt[e], 1);
+    perm[s] = p;
+    pos[p] = s;
+  }
+}
+
+#define GG_T 64
+#define GG_K 16
+
+template <typename T, int SWIGLU>
+__global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(
+    const T* __restrict__ A, const T* __restrict__ Wt, const int* __restrict__ plan, int P, int E,
+    int top, int K, int N, T* __restrict__ out) {
+  __shared__ float As[GG_K][GG_T + 1], Bs[GG_K][GG_T + 1], Bu[SWIGLU ? GG_K : 1][GG_T + 1];
+  const int* offsets = plan;
+  const int* perm = plan + E + 2;
+  // which expert segment and which 64-row tile of it this workgroup owns
+  int tile = blockIdx.x, e = 0, r0 = 0, r1 = 0;
+  for (; e < E; ++e) {
+    const int s0 = offsets[e], s1 = offsets[e + 1];
+    const int nt = (s1 - s0 + GG_T - 1) / GG_T;
+    if (tile < nt) { r0 = s0 + tile * GG_T; r1 = min(s1, r0 + GG_T); break; }
+    tile -= nt;
+  }
+  if (e == E) return;
+  const int n0 = blockIdx.y * GG_T;
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  const int wrows = SWIGLU ? 2 * N : N;        // rows of one expert's weight
+  const T* We = Wt + (size_t)e * wrows * K;
+  float acc[4][4], accu[SWIGLU ? 4 : 1][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { acc[i][j] = 0.f; if (SWIGLU) accu[i][j] = 0.f; }
+  for (int k0 = 0; k0 < K; k0 += GG_K) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < GG_T * GG_K; i += 256) {
+      const int r = i / GG_K, kk = i % GG_K;
+      float a = 0.f, b = 0.f, u = 0.f;
+      if (k0 + kk < K) {
+        if (r0 + r < r1) {
+          const size_t src = SWIGLU ? (size_t)(perm[r0 + r] / top) : (size_t)(r0 + r);
+          a = Act<T>::ld(A + src * K + k0 + kk);
+        }
+        if (n0 + r < N) {
+          b = Act<T>::ld(We + (size_t)(n0 + r) * K + k0 + kk);
+          if (SWIGLU) u = Act<T>::ld(We + (size_t)(N + n0 + r) * K + k0 + kk);
+        }
+      }
+      As[kk][r] = a;
+      Bs[kk][r] = b;
+      if (SWIGLU) Bu[kk][r] = u;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GG_K; ++kk) {
+      float a[4], b[4], u[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = As[kk][ty * 4 + i];
+        b[i] = Bs[kk][tx * 4 + i];
+        if (SWIGLU) u[i] = Bu[kk][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] += a[i] * b[j];
+          if (SWIGLU) accu[i][j] += a[i] * u[j];
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + ty * 4 + i;
+    if (r >= r1) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N)
+        Act<T>::st(out + (size_t)r * N + n, SWIGLU ? silu_f(acc[i][j]) * accu[i][j] : acc[i][j]);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(
+    const T* __restrict__ h, const T* __restrict__ y, const int* __restrict__ idx,
+    const float* __restrict__ wt, const int* __restrict__ plan, int P, int top, int E, int d,
+    float* __restrict__ out) {
+  const int t = blockIdx.x;
+  const int* pos = plan + E + 2 + P;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int p = t * top + k;
+      const float v = idx[p] >= E ? Act<T>::ld(h + (size_t)t * d + c)
+                                  : Act<T>::ld(y + (size_t)pos[p] * d + c);
+      s += wt[p] * v;
+    }
+    out[(size_t)t * d + c] = s;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_any_kernel(const T* __restrict__ x, int F,
+                                                           T* __restrict__ y) {
+  const size_t r = blockIdx.x;
+  for (int c = threadIdx.x; c < F; c += blockDim.x)
+    Act<T>::st(y + r * F + c,
+               silu_f(Act<T>::ld(x + r * 2 * F + c)) * Act<T>::ld(x + r * 2 * F + F + c));
+}
+
+extern "C" int loqa_silu_mul_any(const void* x, int dt, int T, int F, void* y, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (dt == 0)
+    hipLaunchKernelGGL(silu_mul_any_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)x, F,
+                       (bf16_t*)y);
+  else
+    hipLaunchKernelGGL(silu_mul_any_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)x, F,
+                       (float*)y);
+  return (int)hipGetLastError();
+}
+
+extern "C" int loqa_moe_route(const void* z, const void* corr, int E, int G, int keep, int top,
+                              void* idx, void* wt, int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (E > MOE_MAX_E || E <= 0 || G <= 0 || E % G || top <= 0 || top > E)
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(64), 0, st, (const float*)z, (const float*)corr,
+                     E, G, keep, top, (int*)idx, (float*)wt);
+  return (int)hipGetLastError();
+}
+
+extern "C" int loqa_moe_plan(const void* idx, int P, int E, void* plan, hipStream_t st) {
+  if (E > MOE_MAX_E) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(256), 0, st, (const int*)idx, P, E, (int*)plan);
+  return (int)hipGetLastError();
+}
+
+extern "C" int loqa_moe_grouped_gemm(const void* A, int dt, const void* W, const void* plan, int P,
+                                     int E, int top, int K, int N, int swiglu, void* out,
+                                     hipStream_t st) {
+  if (P <= 0) return 0;
+  const dim3 grid((P + GG_T - 1) / GG_T + E, (N + GG_T - 1) / GG_T);
+#define GO(TT, SW)                                                                              \
+  hipLaunchKernelGGL((moe_grouped_gemm_kernel<TT, SW>), grid, dim3(256), 0, st, (const TT*)A,   \
+                     (const TT*)W, (const int*)plan, P, E, top, K, N, (TT*)out)
+  if (dt == 0) { if (swiglu) GO(bf16_t, 1); else GO(bf16_t, 0); }
+  else { if (swiglu) GO(float, 1); else GO(float, 0); }
+#undef GO
+  return (int)hipGetLastError();
+}
+
+extern "C" int loqa_moe_combine(const void* h, const void* y, int dt, const void* idx,
+                                const void* wt, const void* plan, int T, int top, int E, int d,
+                                void* out, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (dt == 0)
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)h,
+                       (const bf16_t*)y, (const int*)idx, (const float*)wt, (const int*)plan, T * top,
+                       top, E, d, (float*)out);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)h,
+                       (const float*)y, (const int*)idx, (const float*)wt, (const int*)plan, T * top,
+                       top, E, d, (float*)out);
+  return (int)hipGetLastError();
+}

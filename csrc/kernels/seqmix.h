@@ -1,0 +1,25 @@
+// Helpers shared by the sequence-mixer kernels of the hybrid decoders
+// (norm_dyt.hip, attn_latent.hip, lightning.hip, moe.hip).
+//
+// Activations are bfloat16 or float32, chosen at run time by a dtype code
+// (0: bf16, 1: f32); every kernel is a template over the storage type and does
+// its arithmetic in f32. Small vectors (norm weights, sinks, decays, router
+// corrections) are always f32.
+#pragma once
+#include "common.h"
+#include <math.h>
+
+template <typename T> struct Act;
+template <> struct Act<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf2f(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f2bf(v); }
+};
+template <> struct Act<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+
+static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -81,19 +81,36 @@ def _build_lib(name: str, sources: list[str], headers: list[str], flags: list[st
     return out
 
 
-def build(force: bool = False, debug: bool = False) -> list[str]:
+# The sequence-mixer kernels of the hybrid decoders are a library of their own:
+# a checkout that only replays or serves such a model compiles these four files
+# (seconds) and not the whole kernel set (minutes).
+SEQMIX_SOURCES = ("norm_dyt.hip", "attn_latent.hip", "lightning.hip", "moe.hip")
+
+# hipcc may not form packed-f32 VALU instructions from scalar float code
+NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build(force: bool = False, debug: bool = False, only=None, quiet: bool = False) -> list[str]:
+    """Build the native libraries (all, or the names in ``only``) in-tree."""
     opt = ["-O0", "-g"] if debug else ["-O3"]
     kflags = [f"--offload-arch={ARCH}", *opt, "-std=c++17", "-munsafe-fp-atomics",
-              f"-I{os.path.join(CSRC, 'kernels')}"]
-    ksrc = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.hip")))
+              f"-I{os.path.join(CSRC, 'kernels')}", *NO_PACKED_F32]
+    allk = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.hip")))
+    ssrc = [p for p in allk if os.path.basename(p) in SEQMIX_SOURCES]
+    ksrc = [p for p in allk if os.path.basename(p) not in SEQMIX_SOURCES]
     khdr = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.h")))
+    shdr = [p for p in khdr if os.path.basename(p) in ("common.h", "seqmix.h")]
     rsrc = sorted(glob.glob(os.path.join(CSRC, "runtime", "*.cpp")))
     rhdr = sorted(glob.glob(os.path.join(CSRC, "runtime", "*.h")))
     rflags = [*opt, "-std=c++17", "-D__HIP_PLATFORM_AMD__"]
-    return [
-        _build_lib("libloqa_kernels.so", ksrc, khdr, kflags, force),
-        _build_lib("libloqa_runtime.so", rsrc, rhdr, rflags, force),
-    ]
+    libs = [("libloqa_kernels.so", ksrc, khdr, kflags),
+            ("libloqa_seqmix.so", ssrc, shdr, kflags),
+            ("libloqa_runtime.so", rsrc, rhdr, rflags)]
+    out = []
+    for name, src, hdr, flags in libs:
+        if only is None or name in only:
+            out.append(_build_lib(name, src, hdr, flags, force))
+    return out
 
 
 def build_sanitized(kind: str = "address,undefined", out_dir: str | None = None) -> str:

@@ -127,6 +127,9 @@ class GrammarTables:
         self.generic_free = int(safe.nonzero()[0])
         self.generic_digit = tok.token_id("0")
         self.generic_digit2 = int(digits2.nonzero()[0]) if self.ROW_DIGIT2 >= 0 else -1
+        # every token allowed: unconstrained requests (FreeRun)
+        self.ROW_ALL = len(rows)
+        rows.append(torch.ones(V, dtype=torch.bool))
         self._rows = rows
         self._tries: dict[tuple, _Trie] = {}
         self._lit_cache: dict[str, list[int]] = {}
@@ -173,6 +176,50 @@ class GrammarTables:
 
     def allowed(self, row: int) -> torch.Tensor:
         return self._rows[row]
+
+
+class FreeRun:
+    """Sampler state of an unconstrained greedy request, with the interface of
+    ``GrammarState``: every token is allowed, nothing is forced, and the run
+    ends after ``max_new`` sampled tokens or at ``stop``. ``tables`` may be
+    None (an engine whose vocabulary has no grammar tables)."""
+
+    def __init__(self, tables: "GrammarTables | None", max_new: int, stop: int | None = None):
+        self.t, self.max_new, self.stop = tables, max(1, int(max_new)), stop
+        self.done = False
+        self.emitted: list[int] = []
+        self.free_steps = 0
+
+    def start(self) -> list[int]:
+        return []
+
+    def mask_row(self) -> int:
+        return self.t.ROW_ALL if self.t is not None else 0
+
+    def advance(self, tok: int) -> list[int]:
+        self.emitted.append(int(tok))
+        self.free_steps += 1
+        if len(self.emitted) >= self.max_new or (self.stop is not None and tok == self.stop):
+            self.done = True
+        return []
+
+    def text(self) -> str:
+        if self.t is None:
+            return " ".join(str(t) for t in self.emitted)
+        return self.t.tok.decode(self.emitted)
+
+    # the pipelined decode speculates on grammar-forced tokens only: a free
+    # run never predicts, so its steps are fed once the sampled token is known
+    def predict(self):
+        return None
+
+    def is_generic(self, tok: int) -> bool:
+        return True
+
+    def fork(self) -> "FreeRun":
+        g = FreeRun(self.t, self.max_new, self.stop)
+        g.done = self.done
+        return g
 
 
 class GrammarState:

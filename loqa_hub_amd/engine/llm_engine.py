@@ -33,7 +33,8 @@ from .. import ops
 from ..models.configs import LlamaConfig
 from .batching import MPAD_PLAN, join_futures, plan_step, plan_step_mpad
 from ..models.llama import LlamaModel, LlamaWeights, StepMeta, TPGroup
-from .grammar import GrammarState, GrammarTables
+from .grammar import FreeRun, GrammarState, GrammarTables
+from .hybrid_cache import HybridCache
 from .kv_cache import PagedKVCache
 from .tokenizer import get_tokenizer
 from ..parallel.custom_allreduce import ERR_TOKEN, CollectiveError
@@ -44,8 +45,12 @@ log = logging.getLogger("loqa.llm")
 @dataclass
 class GenRequest:
     prompt: list[int]
-    schema: list
+    # grammar segments of a constrained decode; None: unconstrained greedy
+    # decoding for ``max_new_tokens`` tokens (or until ``stop_token``)
+    schema: list | None
     seq_id: int = -1
+    max_new_tokens: int = 16
+    stop_token: int | None = None
     # filled by the engine
     grammar: GrammarState | None = None
     feed: list[int] = field(default_factory=list)
@@ -74,49 +79,78 @@ class LLMEngine:
     SEQ_BUCKETS = [1, 2, 4, 8, 16, 32, 64, 128]
     RES_SLOTS = 3       # result ring slots (>= steps in flight + 1)
 
-    def __init__(self, cfg: LlamaConfig, device, *, seed: int = 0, max_seqs: int = 64,
+    def __init__(self, cfg, device, *, seed: int = 0, max_seqs: int = 64,
                  max_seq_len: int = 1024, block_size: int = 16, num_blocks: int | None = None,
                  tp: TPGroup | None = None, use_graphs: bool = True, prefill_chunk: int = 8192,
-                 weights: LlamaWeights | None = None, fused_decode: bool = True,
-                 compact: bool = False, tokenizer=None):
+                 weights=None, fused_decode: bool = True,
+                 compact: bool = False, tokenizer=None, dtype=torch.bfloat16):
+        from ..models.registry import build_model, family_of, random_lm_weights
         self.cfg = cfg
+        # the model family (models/registry.py) decides the weights, the step
+        # function and the kind of cache; scheduling, batching and sampling
+        # below are shared
+        self.family = family_of(cfg)
+        self.hybrid = self.family.hybrid
+        self.dtype = dtype
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
             self.device = torch.device("cuda", torch.cuda.current_device())
         self.tp = tp or TPGroup()
+        if self.hybrid and self.tp.world > 1:
+            raise ValueError(f"{self.family.name}: tensor parallel serving is not available")
         from ..utils.streams import decode_cap, init_pools
         init_pools(self.device)       # fixed stream -> hardware-queue placement
         self.max_wgs = decode_cap("LOQA_LLM_MAX_WGS")
         with ops.decode_cap(self.max_wgs):
-            self.weights = weights or LlamaWeights(cfg, self.device, seed=seed, tp=self.tp,
-                                                   compact=compact)
+            self.weights = weights or random_lm_weights(cfg, self.device, seed=seed, tp=self.tp,
+                                                        compact=compact, dtype=dtype,
+                                                        max_positions=max_seq_len)
         self.weights.max_wgs = self.max_wgs or ops.MAX_DECODE_WGS
-        self.model = LlamaModel(self.weights)
+        self.model = build_model(self.weights)
         # a checkpoint's own tokenizer (tokenizer.HFTokenizer), else the
-        # synthetic one of the random-init weights
-        self.tok = tokenizer or get_tokenizer(cfg.vocab_size)
-        self.grammar = GrammarTables(self.tok, self.device)
-        from .grammar import INTENTS
-        self.grammar.trie(INTENTS)
-        self.grammar.trie(["true", "false"])
-        self.masks = self.grammar.mask_table(self.device)
+        # synthetic one of the random-init weights; a vocabulary too small for
+        # it serves unconstrained (schema-less) requests only
+        self.tok = tokenizer
+        if self.tok is None:
+            try:
+                self.tok = get_tokenizer(cfg.vocab_size)
+            except ValueError:
+                if not self.hybrid:
+                    raise
+        self.grammar = self.masks = None
+        if self.tok is not None:
+            self.grammar = GrammarTables(self.tok, self.device)
+            from .grammar import INTENTS
+            self.grammar.trie(INTENTS)
+            self.grammar.trie(["true", "false"])
+            self.masks = self.grammar.mask_table(self.device)
         self.max_seqs, self.max_seq_len = max_seqs, max_seq_len
         self.block_size = block_size
         self.max_blocks = (max_seq_len + block_size - 1) // block_size
         if num_blocks is None:
             num_blocks = max_seqs * self.max_blocks + 64
-        self.kv = PagedKVCache(cfg.n_layers, self.weights.hkv, cfg.head_dim, num_blocks, block_size,
-                               self.device)
         self.is_gpu = self.device.type == "cuda"
-        # grouped decode attention holds G * q_len <= 32 query rows per kv head
-        self.max_decode_q = max(1, 32 // (self.weights.h // self.weights.hkv))
-        self.attn_ws = ops.AttnWorkspace(self.device, 128, self.weights.h, cfg.head_dim,
-                                         (max_seq_len + 127) // 128) if self.is_gpu else None
+        if self.hybrid:
+            if getattr(self.weights, "max_positions", max_seq_len) < max_seq_len:
+                raise ValueError("the weights' rotary tables are shorter than max_seq_len")
+            # latent pages + state slots on the shared block pool
+            self.kv = HybridCache(self.model.cache_spec(), num_blocks, block_size, max_seqs,
+                                  self.device, dtype)
+            self.max_decode_q = 32
+            self.attn_ws = None
+            use_graphs = fused_decode = False
+        else:
+            self.kv = PagedKVCache(cfg.n_layers, self.weights.hkv, cfg.head_dim, num_blocks,
+                                   block_size, self.device)
+            # grouped decode attention holds G * q_len <= 32 query rows per kv head
+            self.max_decode_q = max(1, 32 // (self.weights.h // self.weights.hkv))
+            self.attn_ws = ops.AttnWorkspace(self.device, 128, self.weights.h, cfg.head_dim,
+                                             (max_seq_len + 127) // 128) if self.is_gpu else None
         # decode-attention keys per split (>= 128: the workspace holds max_seq_len / 128 splits)
         self.attn_split_keys = max(128, int(os.environ.get("LOQA_LLM_ATTN_SPLIT_KEYS", "128")) // 32 * 32)
         self.use_graphs = use_graphs and self.is_gpu
         # fused-epilogue decode GEMMs (single GPU, <= 32 tokens per step)
-        self.fused_decode = fused_decode and self.weights.fused
+        self.fused_decode = fused_decode and getattr(self.weights, "fused", False)
         self.scratch = ops.FusedScratch(self.device)
         self.prefill_chunk = prefill_chunk
         # inline prefill: a new request whose uncached prompt tail is at most
@@ -218,6 +252,9 @@ class LLMEngine:
         max_ctx = max(int(ctx[:B].max()) if B else 1, 1)
         host = {"tokens": tokens, "positions": positions, "slots": slots, "cu_q": cu,
                 "ctx_lens": ctx, "block_tables": bt, "logit_idx": lidx}
+        if self.hybrid:
+            host["state_slots"] = np.asarray(
+                self.kv.state_slots([r.seq_id for r in seqs], B_pad), np.int32)
         return max_q, max_ctx, host
 
     def _to_device(self, host: dict, dst: dict | None = None) -> dict:
@@ -235,6 +272,10 @@ class LLMEngine:
 
     # ------------------------------------------------------------ forward
     def _forward_sample(self, meta: StepMeta, mask_rows: torch.Tensor) -> torch.Tensor:
+        if self.hybrid:
+            # one step function for prompts, decode tokens and mixed batches
+            logits = self.model.forward(meta, self.kv)[: mask_rows.numel()]
+            return ops.masked_argmax(logits, self.masks, mask_rows if self.masks is not None else None)
         if meta.decode:
             if self.fused_decode and meta.tokens.numel() <= 64:
                 logits = self.model.forward_decode_fused(meta, self.kv.k, self.kv.v, self.attn_ws,
@@ -277,7 +318,8 @@ class LLMEngine:
     def _build_meta(self, dev: dict, max_q: int, max_ctx: int, decode: bool) -> StepMeta:
         return StepMeta(tokens=dev["tokens"], positions=dev["positions"], slots=dev["slots"],
                         cu_q=dev["cu_q"], ctx_lens=dev["ctx_lens"], block_tables=dev["block_tables"],
-                        logit_idx=dev["logit_idx"], max_q=max_q, max_ctx=max_ctx, decode=decode)
+                        logit_idx=dev["logit_idx"], max_q=max_q, max_ctx=max_ctx, decode=decode,
+                        state_slots=dev.get("state_slots"))
 
     CTX_BUCKET = 256
 
@@ -410,11 +452,60 @@ class LLMEngine:
         self._graphs_frozen = True
         return n
 
+    # -------------------------------------------------------------- replay
+    def open_sequence(self) -> GenRequest:
+        """Admit an empty sequence that is fed explicitly (``step_logits``):
+        it takes a sequence id, an empty block table and, for models with
+        recurrent layers, a state slot. ``close_sequence`` gives them back."""
+        r = GenRequest([], None)
+        r.seq_id = self._next_id
+        self._next_id += 1
+        if self.kv.pool.add_seq(r.seq_id, []) < 0:
+            raise RuntimeError("duplicate sequence id")
+        return r
+
+    def close_sequence(self, r: GenRequest) -> None:
+        r.done = True
+        self.kv.pool.free_seq(r.seq_id)
+
+    def step_logits(self, seqs: list[GenRequest], feeds: list[list[int]],
+                    want: list[list[int]]) -> torch.Tensor:
+        """One engine step over given tokens, sampling nothing: every
+        sequence's ``feeds[i]`` (a prompt portion or a single token) goes
+        through the model as ONE flat batch on top of what the cache and the
+        state slots hold; returns the f32 logits [sum(len(w)), vocab] at the
+        places ``want[i]`` (indices into ``feeds[i]``), in order. This is the
+        step function the generation paths run (``_meta`` + the model's
+        forward), with the sampling left out."""
+        if not seqs:
+            return torch.zeros(0, self.cfg.vocab_size)
+        max_q, max_ctx, host = self._meta(seqs, feeds, decode=False)
+        cu = host["cu_q"]
+        rows = [int(cu[i]) + int(w) for i, ws in enumerate(want) for w in ws]
+        for i, ws in enumerate(want):
+            if any(not 0 <= int(w) < len(feeds[i]) for w in ws):
+                raise IndexError("a wanted place lies outside its feed")
+        host["logit_idx"] = np.asarray(rows or [0], np.int64)
+        dev = self._to_device(host)
+        meta = self._build_meta(dev, max_q, max_ctx, False)
+        if self.hybrid:
+            logits = self.model.forward(meta, self.kv)
+        else:
+            logits = self.model.logits(self.model.forward(meta, self.kv.k, self.kv.v, self.attn_ws))
+        self.stats["prefill_tokens"] += sum(len(f) for f in feeds)
+        return logits[: len(rows)].float()
+
     # ------------------------------------------------------------ generate
     def submit(self, req: GenRequest) -> GenRequest:
         req.seq_id = self._next_id
         self._next_id += 1
-        req.grammar = GrammarState(self.grammar, req.schema)
+        if req.schema is None:
+            req.grammar = FreeRun(self.grammar, req.max_new_tokens, req.stop_token)
+        elif self.grammar is None:
+            raise ValueError("this engine's vocabulary has no grammar tables: "
+                             "only schema-less requests are served")
+        else:
+            req.grammar = GrammarState(self.grammar, req.schema)
         start = req.grammar.start()
         req.feed = list(req.prompt) + start
         if req.on_tokens is not None and start:
@@ -573,7 +664,10 @@ class LLMEngine:
             self.stats["replay_call_s"] += t15 - t1
             self.stats["gpu_wait_s"] += t2 - t1
         else:
-            max_q, max_ctx, host = self._meta(live, feeds, True, B, ops.mpad_for(T))
+            # (the fused Llama GEMMs want padded row counts; the hybrid step
+            # function takes the batch as it is)
+            max_q, max_ctx, host = self._meta(live, feeds, True, B,
+                                              T if self.hybrid else ops.mpad_for(T))
             host["mask_rows"] = rows
             dev = self._to_device(host)
             meta = self._build_meta(dev, max_q, max_ctx, True)
@@ -868,6 +962,8 @@ class LLMEngine:
         leading live sequences + flash prefill for the prompt chunks (adds
         ``cu_tail`` to ``host``), else None."""
         nd = sum(1 for k in kinds if k == 0)
+        if self.hybrid:
+            return None      # one attention launch serves decode rows and chunks
         if (not self.MIXED_SPLIT or nd == 0 or nd == len(kinds)
                 or any(k != 0 for k in kinds[:nd])):
             return None

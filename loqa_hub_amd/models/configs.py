@@ -215,3 +215,114 @@ def checkpoint_config(path: str):
         return None
     with open(f, encoding="utf-8") as fh:
         return json.load(fh)
+
+
+# --------------------------------------------------------------------------
+# Pipizen: a hybrid decoder whose config.json lists its layers one by one.
+# Every size and constant is taken from that file (or a tensor's shape).
+@dataclass(frozen=True)
+class RotaryConfig:
+    dims: int                       # rotated entries (pairs 2i, 2i+1), <= rot_dim
+    base: float
+    yarn: tuple | None = None       # (factor, original, fast, slow)
+
+
+@dataclass(frozen=True)
+class LatentAttnConfig:
+    heads: int
+    dim: int                        # unrotated query/key size per head
+    rot_dim: int                    # rotated query/key size per head (key part shared)
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot: RotaryConfig
+    kv_from: int | None = None      # reuse that layer's latent cache
+
+
+@dataclass(frozen=True)
+class LightningConfig:
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+
+
+@dataclass(frozen=True)
+class FeedForwardConfig:
+    kind: str                       # "dense" | "moe"
+    ff: int = 0                     # dense width / expert width
+    experts: int = 0
+    identity: int = 0               # trailing router outputs that pass the input through
+    top: int = 0
+    groups: int = 1
+    keep: int = 1
+    shared_ff: int = 0              # 0: no shared expert
+
+
+@dataclass(frozen=True)
+class HybridLayerConfig:
+    kind: str                       # "latent_attention" | "lightning"
+    mixer: object
+    mlp: FeedForwardConfig | None
+
+
+@dataclass(frozen=True)
+class PipizenConfig:
+    name: str
+    vocab_size: int
+    d_model: int
+    norm_eps: float
+    layers: tuple
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+
+def pipizen_config_from_json(d: dict, name: str = "pipizen") -> PipizenConfig:
+    layers = []
+    for i, L in enumerate(d["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind == "latent_attention":
+            r = m["rot"]
+            sc = r.get("scaling")
+            rot = RotaryConfig(int(r["dims"]), float(r["base"]),
+                               (float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                                float(sc["slow"])) if sc else None)
+            src = m.get("kv_from")
+            mixer = LatentAttnConfig(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]),
+                                     int(m["vdim"]), int(m["kv_rank"]), float(m["scale"]), rot,
+                                     None if src is None else int(src))
+            if mixer.kv_from is not None and not 0 <= mixer.kv_from < i:
+                raise ValueError(f"layer {i}: kv_from {mixer.kv_from} is not an earlier layer")
+        elif kind == "lightning":
+            mixer = LightningConfig(int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                                    tuple(float(v) for v in m["decay"]))
+            if len(mixer.decay) != mixer.heads:
+                raise ValueError(f"layer {i}: one decay per head expected")
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = L.get("mlp")
+        if not f:
+            mlp = None
+        elif f["kind"] == "dense":
+            mlp = FeedForwardConfig("dense", int(f["ff"]))
+        elif f["kind"] == "moe":
+            r = f["router"]
+            g = r.get("groups") or {}
+            mlp = FeedForwardConfig("moe", int(f["expert"]["ff"]), int(r["experts"]),
+                                    int(r.get("identity", 0)), int(r["top"]),
+                                    int(g.get("count", 1)), int(g.get("keep", g.get("count", 1))),
+                                    int((f.get("shared") or {}).get("ff", 0)))
+            if (mlp.experts + mlp.identity) % mlp.groups:
+                raise ValueError(f"layer {i}: router outputs do not split into {mlp.groups} groups")
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(HybridLayerConfig(kind, mixer, mlp))
+    for i, L in enumerate(layers):
+        if L.kind == "latent_attention" and L.mixer.kv_from is not None:
+            s = layers[L.mixer.kv_from]
+            if s.kind != "latent_attention" or s.mixer.kv_from is not None:
+                raise ValueError(f"layer {i}: kv_from must name a latent layer with its own cache")
+    return PipizenConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
+                         tuple(layers))

@@ -45,6 +45,8 @@ class StepMeta:
     # their own attention launches (grouped decode attention reads each kv
     # head's cache once; the flash prefill kernel would re-read it per q head)
     split: tuple | None = None
+    # state slot of each sequence (models with recurrent layers), int32 [B]
+    state_slots: torch.Tensor | None = None
 
 
 class TPGroup:

@@ -424,3 +424,33 @@ def load_vits(path: str, device, cfg=None):
         with open(vf, encoding="utf-8") as fh:
             vocab = json.load(fh)
     return cfg, vits_from_state_dict(cfg, sd, device), vocab
+
+
+# -------------------------------------------------------------------- Pipizen
+def read_safetensors_raw(path: str) -> dict[str, torch.Tensor]:
+    """All tensors of a checkpoint on the host in their stored dtypes
+    (memory-mapped read; integer tables stay integers)."""
+    from safetensors import safe_open
+    out: dict[str, torch.Tensor] = {}
+    for f in _files(path):
+        with safe_open(f, framework="pt", device="cpu") as st:
+            for name in st.keys():
+                out[name] = st.get_tensor(name)
+    return out
+
+
+def load_pipizen(cfg, path: str, device, dtype=torch.bfloat16, max_positions: int = 8192):
+    """A Pipizen checkpoint (its own tensor naming) in the fused device layout;
+    ``dtype`` is the activation / matrix dtype (bfloat16 serving, float32 exact)."""
+    from .pipizen import PipizenWeights
+    return PipizenWeights(cfg, read_safetensors_raw(path), device, dtype, max_positions)
+
+
+def save_pipizen(cfg, state: dict[str, torch.Tensor], folder: str) -> None:
+    """Write ``state`` (checkpoint naming) and the config.json of ``cfg``."""
+    import json
+    from .pipizen import config_to_json
+    os.makedirs(folder, exist_ok=True)
+    write_safetensors(state, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(config_to_json(cfg), f, indent=1)

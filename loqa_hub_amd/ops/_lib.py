@@ -205,6 +205,24 @@ _RUNTIME_SIGS = {
 }
 
 
+_vp, _i, _f, _l = c_void_p, c_int, c_float, c_ll
+_SEQMIX_SIGS = {
+    "loqa_dyt_norm": [_vp, _i, _vp, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+    "loqa_dyt_add_norm": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+    "loqa_latent_append": [_vp, _i, _l, _vp, _f, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _i, _vp],
+    "loqa_latent_attention": [_vp, _l, _l, _vp, _l, _l, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp,
+                              _i, _vp, _f, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp],
+    "loqa_lightning_scan": [_vp, _i, _l, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "loqa_gated_rmsnorm": [_vp, _vp, _vp, _i, _l, _f, _vp, _i, _i, _i, _vp],
+    "loqa_silu_mul_any": [_vp, _i, _i, _i, _vp, _vp],
+    "loqa_moe_route": [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp],
+    "loqa_moe_plan": [_vp, _i, _i, _vp, _vp],
+    "loqa_moe_grouped_gemm": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp],
+    "loqa_moe_combine": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
+}
+_seqmix = None
+
+
 class NativeLibraryMissing(RuntimeError):
     pass
 
@@ -217,7 +235,18 @@ def _load(name: str) -> ctypes.CDLL:
     return ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
 
 
-def kernels() -> ctypes.CDLL:
+_dispatch = None
+
+
+def kernels():
+    """The kernel entry points (both kernel libraries, each loaded on first use)."""
+    global _dispatch
+    if _dispatch is None:
+        _dispatch = _Kernels()
+    return _dispatch
+
+
+def _main_kernels() -> ctypes.CDLL:
     global _kernels
     if _kernels is None:
         with _lock:
@@ -235,6 +264,34 @@ def kernels() -> ctypes.CDLL:
     return _kernels
 
 
+class _Kernels:
+    """Attribute lookup over the kernel libraries: the sequence-mixer entry
+    points live in ``libloqa_seqmix.so``, everything else in
+    ``libloqa_kernels.so`` (loaded only when one of its kernels is called)."""
+
+    def __getattr__(self, name: str):
+        if name in _SEQMIX_SIGS:
+            fn = getattr(seqmix(), name)
+        else:
+            fn = getattr(_main_kernels(), name)
+        setattr(self, name, fn)
+        return fn
+
+
+def seqmix() -> ctypes.CDLL:
+    global _seqmix
+    if _seqmix is None:
+        with _lock:
+            if _seqmix is None:
+                lib = _load("libloqa_seqmix.so")
+                for fn, sig in _SEQMIX_SIGS.items():
+                    f = getattr(lib, fn)
+                    f.argtypes = sig
+                    f.restype = c_int
+                _seqmix = lib
+    return _seqmix
+
+
 def runtime() -> ctypes.CDLL:
     global _runtime
     if _runtime is None:
@@ -249,9 +306,16 @@ def runtime() -> ctypes.CDLL:
     return _runtime
 
 
+def load_all() -> None:
+    """Load every native library (a missing one raises)."""
+    _main_kernels()
+    seqmix()
+    runtime()
+
+
 def available() -> bool:
     try:
-        kernels()
+        _main_kernels()
         return True
     except (NativeLibraryMissing, OSError):
         return False

@@ -593,3 +593,177 @@ def whisper_decoder_ref(w, tokens: list[int], enc: torch.Tensor) -> torch.Tensor
         x = x + lin(gelu(lin(ln(x, L["ln2_w"], L["ln2_b"]), L["fc1"], L["fc1_b"])), L["fc2"],
                     L["fc2_b"])
     return ln(x, w.dec_ln_w, w.dec_ln_b) @ w.tok_embed.float().t()
+
+
+# ---------------------------------------------------------------------------
+# Sequence-mixer building blocks of the hybrid decoders (models/pipizen.py):
+# Dynamic-Tanh norm, interleaved rotary tables with YaRN, latent (compressed
+# KV) attention with a softmax sink, decayed linear attention with a carried
+# state, and a grouped top-k expert router. Everything the recurrences and the
+# softmax touch is f32; ``out_dtype`` is the activation dtype of the caller.
+def dyt_norm(x, w, b, alpha: float, out_dtype, row_idx=None):
+    """tanh(alpha x) * w + b (no mean, no variance)."""
+    if row_idx is not None:
+        x = x.index_select(0, row_idx.long())
+    return (torch.tanh(x.float() * alpha) * w.float() + b.float()).to(out_dtype)
+
+
+def dyt_add_norm(resid, y, post, nxt, out_dtype):
+    """resid (f32, in place) += dyt(y; post); returns dyt(resid; nxt) or None."""
+    resid.add_(dyt_norm(y, post[0], post[1], post[2], torch.float32))
+    if nxt is None:
+        return None
+    return dyt_norm(resid, nxt[0], nxt[1], nxt[2], out_dtype)
+
+
+def rope_table_pairs(dims: int, max_pos: int, base: float, yarn: tuple | None = None,
+                     device=None) -> torch.Tensor:
+    """[max_pos, dims/2, 2] f32 (cos, sin) for the interleaved layout (entry 2i
+    rotates with entry 2i+1). ``yarn`` = (factor, original, fast, slow): each
+    frequency is a blend of itself and itself / factor, the blend ramping
+    between the dimensions whose wavelength fits the original context ``fast``
+    and ``slow`` times; cos and sin carry the magnitude 0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    mag = 1.0
+    if yarn is not None:
+        factor, orig, fast, slow = (float(v) for v in yarn)
+
+        def turn(t):   # the dimension index whose wavelength makes t turns in the original context
+            return dims * math.log(orig / (2 * math.pi * t)) / (2 * math.log(base))
+        lo = max(math.floor(turn(fast)), 0)
+        hi = min(math.ceil(turn(slow)), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None, :]
+    return (torch.stack([ang.cos(), ang.sin()], dim=-1) * mag).float().to(device)
+
+
+def rotate_pairs(x, cs, dims: int):
+    """x [T, ..., n] (any float) -> f32 copy whose first ``dims`` entries are
+    rotated pairwise by cs [T, dims/2, 2]."""
+    out = x.float().clone()
+    u, v = out[..., 0:dims:2].clone(), out[..., 1:dims:2].clone()
+    c, s = cs[..., 0], cs[..., 1]
+    while c.dim() < u.dim():
+        c, s = c.unsqueeze(1), s.unsqueeze(1)
+    out[..., 0:dims:2] = u * c - v * s
+    out[..., 1:dims:2] = v * c + u * s
+    return out
+
+
+def latent_append(z, norm_w, eps: float, positions, cos_sin, cache, slots, R: int, dims: int):
+    """z [T, R + Dr]: the first R entries RMS-normed (weight ``norm_w``) are
+    the latent, the rest the shared rotary key part; both go to the paged
+    cache [blocks, BLK, R + Dr] at ``slots`` (-1: padding row)."""
+    zf = z.float()
+    c = zf[:, :R]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = rotate_pairs(zf[:, R:], cos_sin[positions.long()], dims)
+    row = torch.cat([c, kr], dim=-1).to(cache.dtype)
+    sl = slots.long()
+    ok = sl >= 0
+    blk = cache.shape[1]
+    cache[(sl // blk)[ok], (sl % blk)[ok]] = row[ok]
+
+
+def latent_attention(qa, qr, cache, cu_q, ctx_lens, block_tables, positions, cos_sin, sink,
+                     scale: float, R: int, dims: int, out):
+    """Causal attention of one shared key/value stream per token (the cached
+    latent row): score = (qa . c + rot(qr) . k_rot) * scale, softmax whose
+    denominator also holds exp(sink[h]); out[h, t] = sum_j p_j c_j.
+    qa [H, T, R], qr [T, H, Dr] (unrotated), out [H, T, R]."""
+    H = qa.shape[0]
+    blk = cache.shape[1]
+    cu = cu_q.tolist()
+    qrot = rotate_pairs(qr, cos_sin[positions.long()], dims)          # [T, H, Dr] f32
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        L = int(ctx_lens[b])
+        idx = torch.arange(L, device=cache.device)
+        rows = cache[block_tables[b].long()[idx // blk], idx % blk].float()   # [L, R + Dr]
+        s = torch.einsum("htr,lr->htl", qa[:, q0:q1].float(), rows[:, :R])
+        s = (s + torch.einsum("thr,lr->htl", qrot[q0:q1], rows[:, R:])) * scale
+        qpos = positions[q0:q1].long()
+        s = s.masked_fill(idx[None, None, :] > qpos[None, :, None], float("-inf"))
+        if sink is not None:
+            s = torch.cat([s, sink.float()[:, None, None].expand(H, q1 - q0, 1)], dim=-1)
+        p = torch.softmax(s, dim=-1)[..., :L]
+        out[:, q0:q1] = torch.einsum("htl,lr->htr", p, rows[:, :R]).to(out.dtype)
+    return out
+
+
+def lightning_scan(qkv, H: int, D: int, Dv: int, state, state_slots, cu_q, positions, decay):
+    """Decayed linear attention, token by token: S <- decay_h S + k v^T,
+    o = S^T q with q, k, v = silu of the [q | k | v] columns of ``qkv``. The
+    state [slots, H, D, Dv] (f32) is read at the sequence's slot (zero when
+    the step's first position is 0) and written back. Returns o f32 [T, H Dv]."""
+    T = qkv.shape[0]
+    a = torch.nn.functional.silu(qkv[:, :2 * H * D + H * Dv].float())
+    q, k = a[:, :H * D].view(T, H, D), a[:, H * D:2 * H * D].view(T, H, D)
+    v = a[:, 2 * H * D:].view(T, H, Dv)
+    o = torch.zeros(T, H, Dv, dtype=torch.float32, device=qkv.device)
+    cu = cu_q.tolist()
+    lam = decay.float()[:, None, None]
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        slot = int(state_slots[b])
+        S = torch.zeros_like(state[slot]) if int(positions[q0]) == 0 else state[slot].clone()
+        for t in range(q0, q1):
+            S = lam * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hde,hd->he", S, q[t])
+        state[slot] = S
+    return o.view(T, H * Dv)
+
+
+def gated_rmsnorm(o, w, gate, eps: float, out_dtype):
+    """rmsnorm(o) * w * sigmoid(gate), the row normalised as a whole."""
+    of = o.float()
+    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def moe_route(z, correction, n_groups: int, keep: int, top: int):
+    """z f32 [T, E] router logits -> (expert index int32 [T, top], weight f32
+    [T, top]). Scores are softmax(z); experts are chosen by score + correction
+    among the ``keep`` best of ``n_groups`` equal groups of neighbours (a
+    group's rank is its best choice score); the weights are the plain scores."""
+    s = torch.softmax(z.float(), dim=-1)
+    choice = s if correction is None else s + correction.float()
+    if n_groups > 1 and keep < n_groups:
+        T, E = s.shape
+        per = E // n_groups
+        gs = choice.view(T, n_groups, per).max(-1).values
+        kept = gs.topk(keep, dim=-1).indices
+        ok = torch.zeros(T, n_groups, dtype=torch.bool, device=z.device).scatter_(1, kept, True)
+        choice = choice.masked_fill(~ok.repeat_interleave(per, dim=1), float("-inf"))
+    idx = choice.topk(top, dim=-1).indices
+    return idx.to(torch.int32), s.gather(1, idx)
+
+
+def moe_experts(h, idx, wt, w_gate_up, w_down, out_dtype):
+    """Weighted sum of each token's chosen experts: expert e < E is the gated
+    feed-forward (w_gate_up [E, 2F, d] = gate | up rows, w_down [E, d, F]);
+    an index >= E is an identity expert (its output is h). Returns f32 [T, d];
+    the expert outputs are rounded to ``out_dtype`` first, as GEMM outputs."""
+    T, d = h.shape
+    E = w_gate_up.shape[0]
+    F = w_gate_up.shape[1] // 2
+    out = torch.zeros(T, d, dtype=torch.float32, device=h.device)
+    for k in range(idx.shape[1]):
+        e = idx[:, k].long()
+        ident = e >= E
+        out += torch.where(ident[:, None], wt[:, k:k + 1] * h.float(), torch.zeros_like(out))
+        for ee in e[~ident].unique().tolist():
+            rows = (e == ee).nonzero()[:, 0]
+            x = h[rows].to(out_dtype)
+            gu = torch.nn.functional.linear(x, w_gate_up[ee])
+            a = (torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()).to(out_dtype)
+            y = torch.nn.functional.linear(a, w_down[ee])
+            out[rows] += wt[rows, k:k + 1] * y.float()
+    return out

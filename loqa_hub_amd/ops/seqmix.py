@@ -1,0 +1,271 @@
+"""Entry points of the sequence-mixer ops of the hybrid decoders: Dynamic-Tanh
+norm, latent (compressed-KV) attention with a softmax sink over a paged latent
+cache, decayed linear attention with a carried per-sequence state, and the
+grouped top-k expert router with its expert feed-forward.
+
+As everywhere in ``ops``: GPU tensors run the HIP kernels
+(``csrc/kernels/norm_dyt.hip``, ``attn_latent.hip``, ``lightning.hip``,
+``moe.hip``), CPU tensors the f32 PyTorch references (the CPU test tier and the
+numerics oracle of the GPU tests). Activations are bfloat16 or float32
+(``_DT``); the residual stream, scores, softmax, recurrent state, router and
+norm statistics are f32 in both.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import reference as ref
+from ._lib import check, kernels, ptr, stream_ptr
+
+_DT = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"activation dtype {t.dtype} is not supported") from None
+
+
+def _f32c(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        raise TypeError(f"{name} must be contiguous float32")
+
+
+def _i32c(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise TypeError(f"{name} must be contiguous int32")
+
+
+class DytParams:
+    """One Dynamic-Tanh norm: f32 weight and bias vectors and the scalar alpha."""
+    __slots__ = ("w", "b", "alpha")
+
+    def __init__(self, w: torch.Tensor, b: torch.Tensor, alpha: float):
+        self.w, self.b, self.alpha = w.float().contiguous(), b.float().contiguous(), float(alpha)
+
+    def tup(self):
+        return self.w, self.b, self.alpha
+
+
+def dyt_norm(x: torch.Tensor, p: DytParams, out_dtype, row_idx: torch.Tensor | None = None
+             ) -> torch.Tensor:
+    """y = tanh(alpha x) * w + b over rows of x [rows, d] (f32 or an activation
+    dtype); ``row_idx`` (int64) gathers rows in the same launch."""
+    if not x.is_cuda:
+        return ref.dyt_norm(x, p.w, p.b, p.alpha, out_dtype, row_idx)
+    assert x.dim() == 2 and x.is_contiguous()
+    d = x.shape[1]
+    rows = x.shape[0] if row_idx is None else row_idx.numel()
+    if row_idx is not None:
+        assert row_idx.dtype == torch.int64 and row_idx.is_contiguous()
+    assert p.w.numel() == d and p.b.numel() == d
+    y = torch.empty(rows, d, dtype=out_dtype, device=x.device)
+    if rows:
+        check(kernels().loqa_dyt_norm(ptr(x), _dt(x), ptr(row_idx), ptr(p.w), ptr(p.b), p.alpha,
+                                      ptr(y), _dt(y), rows, d, stream_ptr(x)), "dyt_norm")
+    return y
+
+
+def dyt_add_norm(resid: torch.Tensor, y: torch.Tensor, post: DytParams,
+                 nxt: DytParams | None, out_dtype) -> torch.Tensor | None:
+    """The fused residual step: resid (f32, in place) += dyt(y; post), and in
+    the same launch h = dyt(resid; nxt) for the next sublayer (None: no h)."""
+    if not resid.is_cuda:
+        return ref.dyt_add_norm(resid, y, post.tup(), None if nxt is None else nxt.tup(), out_dtype)
+    _f32c(resid, "resid")
+    assert y.shape == resid.shape and y.is_contiguous()
+    rows, d = resid.shape
+    h = torch.empty(rows, d, dtype=out_dtype, device=resid.device) if nxt is not None else None
+    if rows:
+        check(kernels().loqa_dyt_add_norm(
+            ptr(resid), ptr(y), _dt(y), ptr(post.w), ptr(post.b), post.alpha,
+            ptr(nxt.w) if nxt else None, ptr(nxt.b) if nxt else None, nxt.alpha if nxt else 0.0,
+            ptr(h), _dt(h) if h is not None else 0, rows, d, stream_ptr(resid)), "dyt_add_norm")
+    return h
+
+
+def rope_table_pairs(dims: int, max_pos: int, base: float, yarn: tuple | None = None,
+                     device=None) -> torch.Tensor:
+    """(cos, sin) table of the interleaved rotary layout, optionally YaRN-scaled
+    (see :func:`reference.rope_table_pairs`); built once at load time."""
+    return ref.rope_table_pairs(dims, max_pos, base, yarn, device)
+
+
+def latent_append(z: torch.Tensor, norm_w: torch.Tensor, eps: float, positions: torch.Tensor,
+                  cos_sin: torch.Tensor, cache: torch.Tensor, slots: torch.Tensor, R: int,
+                  dims: int) -> None:
+    """RMS-norm the latent part of z [T, R + Dr], rotate its rotary key part and
+    store both in the paged latent cache [blocks, BLK, R + Dr] (one launch)."""
+    if not z.is_cuda:
+        return ref.latent_append(z, norm_w, eps, positions, cos_sin, cache, slots, R, dims)
+    T, W = z.shape
+    assert z.stride(1) == 1 and cache.is_contiguous() and cache.dtype == z.dtype
+    assert cache.shape[2] == W and 0 < R <= W and dims % 2 == 0 and dims <= W - R
+    _f32c(norm_w, "norm_w"); _f32c(cos_sin, "cos_sin"); _i32c(positions, "positions")
+    _i32c(slots, "slots")
+    assert norm_w.numel() == R and cos_sin.shape[1] * 2 == dims
+    assert positions.numel() >= T and slots.numel() >= T
+    if T:
+        check(kernels().loqa_latent_append(
+            ptr(z), _dt(z), z.stride(0), ptr(norm_w), eps, ptr(positions), ptr(cos_sin),
+            cos_sin.shape[0], ptr(cache), cache.shape[1], cache.shape[0], ptr(slots), T, R, W - R,
+            dims, stream_ptr(z)), "latent_append")
+
+
+def latent_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Tensor, cu_q: torch.Tensor,
+                     ctx_lens: torch.Tensor, block_tables: torch.Tensor, positions: torch.Tensor,
+                     cos_sin: torch.Tensor, sink: torch.Tensor | None, scale: float, R: int,
+                     dims: int, max_ctx: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Causal attention over the paged latent cache, all heads sharing each
+    cached row: score = (qa . c + rot(qr) . k_rot) * scale; softmax with
+    ``sink`` [H] (f32, optional) in the denominator; out = sum_j p_j c_j.
+    qa [H, T, R] (queries already folded into latent space), qr [T, H, Dr]
+    (unrotated; may be a strided view), out [H, T, R]."""
+    H, T, _ = qa.shape
+    if out is None:
+        out = torch.empty(H, T, R, dtype=qa.dtype, device=qa.device)
+    if not qa.is_cuda:
+        return ref.latent_attention(qa, qr, cache, cu_q, ctx_lens, block_tables, positions,
+                                    cos_sin, sink, scale, R, dims, out)
+    Dr = cache.shape[2] - R
+    assert qa.shape[2] == R and qa.stride(2) == 1 and qr.shape == (T, H, Dr) and qr.stride(2) == 1
+    assert qa.dtype == cache.dtype == qr.dtype == out.dtype and cache.is_contiguous()
+    assert out.is_contiguous() and out.shape == (H, T, R)
+    _i32c(cu_q, "cu_q"); _i32c(ctx_lens, "ctx_lens"); _i32c(block_tables, "block_tables")
+    _i32c(positions, "positions"); _f32c(cos_sin, "cos_sin")
+    if sink is not None:
+        _f32c(sink, "sink")
+        assert sink.numel() == H
+    B = ctx_lens.numel()
+    assert cu_q.numel() == B + 1 and block_tables.shape[0] == B and positions.numel() >= T
+    # few query rows over a long context: split the keys over workgroups
+    hg = (H + 3) // 4
+    ns = 1 if T * hg >= 512 else max(1, min(32, -(-int(max_ctx) // 256), 1024 // max(1, T * hg)))
+    ws = torch.empty(ns * T * H * (R + 2), dtype=torch.float32, device=qa.device) if ns > 1 else None
+    if T:
+        check(kernels().loqa_latent_attention(
+            ptr(qa), qa.stride(1), qa.stride(0), ptr(qr), qr.stride(0), qr.stride(1), _dt(qa),
+            ptr(cache), cache.shape[1], cache.shape[0], ptr(cu_q), ptr(ctx_lens), ptr(block_tables),
+            block_tables.shape[1], ptr(positions), ptr(cos_sin), cos_sin.shape[0], ptr(sink),
+            float(scale), B, H, T, R, Dr, dims, ptr(out), ns, ptr(ws), stream_ptr(qa)),
+            "latent_attention")
+    return out
+
+
+def lightning_scan(qkv: torch.Tensor, H: int, D: int, Dv: int, state: torch.Tensor,
+                   state_slots: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor,
+                   decay: torch.Tensor) -> torch.Tensor:
+    """Decayed linear attention over a flat token batch: per sequence and head
+    S <- decay_h S + k v^T, o = S^T q, token by token in f32, with q, k, v the
+    SiLU of the first columns of ``qkv`` [T, >= 2 H D + H Dv]. ``state`` [slots,
+    H, D, Dv] f32 carries S between steps (a sequence whose first position in
+    this step is 0 starts from zero). Returns o f32 [T, H Dv]. Prompt portions
+    and single decode tokens take the same kernel and the same order of
+    operations, so the result does not depend on how a prompt was cut."""
+    if not qkv.is_cuda:
+        return ref.lightning_scan(qkv, H, D, Dv, state, state_slots, cu_q, positions, decay)
+    T = qkv.shape[0]
+    assert qkv.stride(1) == 1 and qkv.shape[1] >= 2 * H * D + H * Dv
+    _f32c(state, "state"); _f32c(decay, "decay")
+    assert state.shape[1:] == (H, D, Dv) and decay.numel() == H
+    _i32c(state_slots, "state_slots"); _i32c(cu_q, "cu_q"); _i32c(positions, "positions")
+    B = state_slots.numel()
+    assert cu_q.numel() == B + 1
+    o = torch.empty(T, H * Dv, dtype=torch.float32, device=qkv.device)
+    if T:
+        check(kernels().loqa_lightning_scan(
+            ptr(qkv), _dt(qkv), qkv.stride(0), H, D, Dv, ptr(state), state.shape[0],
+            ptr(state_slots), ptr(cu_q), ptr(positions), ptr(decay), ptr(o), B, T,
+            stream_ptr(qkv)), "lightning_scan")
+    return o
+
+
+def gated_rmsnorm(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, eps: float,
+                  out_dtype) -> torch.Tensor:
+    """y = rmsnorm(o) * w * sigmoid(gate) over whole rows of o f32 [T, n];
+    ``gate`` [T, n] may be a column slice of a wider projection."""
+    if not o.is_cuda:
+        return ref.gated_rmsnorm(o, w, gate, eps, out_dtype)
+    _f32c(o, "o"); _f32c(w, "w")
+    T, n = o.shape
+    assert gate.shape == (T, n) and gate.stride(1) == 1 and w.numel() == n
+    y = torch.empty(T, n, dtype=out_dtype, device=o.device)
+    if T:
+        check(kernels().loqa_gated_rmsnorm(ptr(o), ptr(w), ptr(gate), _dt(gate), gate.stride(0), eps,
+                                           ptr(y), _dt(y), T, n, stream_ptr(o)), "gated_rmsnorm")
+    return y
+
+
+def silu_mul_any(x: torch.Tensor) -> torch.Tensor:
+    """[gate | up] -> silu(gate) * up for bf16 or f32 activations."""
+    if not x.is_cuda:
+        return ref.silu_mul(x)
+    assert x.dim() == 2 and x.is_contiguous() and x.shape[1] % 2 == 0
+    T, F2 = x.shape
+    y = torch.empty(T, F2 // 2, dtype=x.dtype, device=x.device)
+    if T:
+        check(kernels().loqa_silu_mul_any(ptr(x), _dt(x), T, F2 // 2, ptr(y), stream_ptr(x)),
+              "silu_mul_any")
+    return y
+
+
+def moe_route(z: torch.Tensor, correction: torch.Tensor | None, n_groups: int, keep: int,
+              top: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Router decisions from f32 logits z [T, E]: softmax scores, choice by
+    score + ``correction`` limited to the ``keep`` best of ``n_groups`` groups of
+    neighbouring experts, weights = the plain scores (not renormalised).
+    Returns (idx int32 [T, top], weight f32 [T, top])."""
+    if not z.is_cuda:
+        return ref.moe_route(z, correction, n_groups, keep, top)
+    _f32c(z, "z")
+    T, E = z.shape
+    assert E % max(1, n_groups) == 0 and 0 < top <= E and E <= 1024
+    if correction is not None:
+        _f32c(correction, "correction")
+        assert correction.numel() == E
+    idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
+    wt = torch.empty(T, top, dtype=torch.float32, device=z.device)
+    if T:
+        check(kernels().loqa_moe_route(ptr(z), ptr(correction), E, max(1, n_groups),
+                                       min(keep, max(1, n_groups)), top, ptr(idx), ptr(wt), T,
+                                       stream_ptr(z)), "moe_route")
+    return idx, wt
+
+
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor, w_gate_up: torch.Tensor,
+                w_down: torch.Tensor) -> torch.Tensor:
+    """Weighted sum of every token's chosen experts, f32 [T, d]. Experts below
+    E = w_gate_up.shape[0] are gated feed-forwards (w_gate_up [E, 2F, d] with
+    gate rows then up rows, w_down [E, d, F]); an index >= E is an identity
+    expert. On the GPU: a device-side plan (tokens grouped by expert, no host
+    round trip), a grouped gate|up GEMM with the SwiGLU epilogue, a grouped
+    down GEMM, and a combine launch that applies the weights in f32."""
+    if not h.is_cuda:
+        return ref.moe_experts(h, idx, wt, w_gate_up, w_down, h.dtype)
+    T, d = h.shape
+    E, F2, _ = w_gate_up.shape
+    F = F2 // 2
+    top = idx.shape[1]
+    assert h.is_contiguous() and w_gate_up.is_contiguous() and w_down.is_contiguous()
+    assert w_gate_up.dtype == h.dtype == w_down.dtype and w_down.shape == (E, d, F)
+    _i32c(idx, "idx"); _f32c(wt, "wt")
+    dev = h.device
+    P = T * top
+    out = torch.empty(T, d, dtype=torch.float32, device=dev)
+    if T == 0:
+        return out
+    # plan: offsets[E + 1] of each expert's segment, perm[P] pair ids sorted by
+    # expert (identity pairs last, past offsets[E]), pos[P] = where each pair sits
+    plan = torch.empty(E + 2 + 2 * P, dtype=torch.int32, device=dev)
+    act = torch.empty(P, F, dtype=h.dtype, device=dev)
+    y = torch.empty(P, d, dtype=h.dtype, device=dev)
+    k, st = kernels(), stream_ptr(h)
+    check(k.loqa_moe_plan(ptr(idx), P, E, ptr(plan), st), "moe_plan")
+    check(k.loqa_moe_grouped_gemm(ptr(h), _dt(h), ptr(w_gate_up), ptr(plan), P, E, top, d, F, 1,
+                                  ptr(act), st), "moe_gate_up")
+    check(k.loqa_moe_grouped_gemm(ptr(act), _dt(h), ptr(w_down), ptr(plan), P, E, top, F, d, 0,
+                                  ptr(y), st), "moe_down")
+    check(k.loqa_moe_combine(ptr(h), ptr(y), _dt(h), ptr(idx), ptr(wt), ptr(plan), T, top, E, d,
+                             ptr(out), st), "moe_combine")
+    return out
