@@ -416,7 +416,19 @@ def main(argv=None) -> int:
     ap.add_argument("--tts-model", default="vits-ljs")
     ap.add_argument("--served-dp", action="store_true",
                     help="--mode hub: serve through the DP front end + worker processes at any N")
+    ap.add_argument("--lm-bench", action="store_true",
+                    help="instead of the hub workload: prefill / decode throughput of the language-"
+                         "model families (Pipizen beside Llama stacks of equal size, random weights)")
+    ap.add_argument("--lm-sizes", default="1b,7b", help="--lm-bench: layer sizes (1b, 7b, tiny)")
+    ap.add_argument("--lm-prompt", type=int, default=2048, help="--lm-bench: prompt tokens")
+    ap.add_argument("--lm-batch", type=int, default=8, help="--lm-bench: decoding sequences")
+    ap.add_argument("--lm-steps", type=int, default=16, help="--lm-bench: timed decode steps")
     args = ap.parse_args(argv)
+    if args.lm_bench:
+        from loqa_hub_amd.engine import lm_bench
+        if args.cpu_smoke:
+            args.lm_sizes = "tiny"
+        return lm_bench.run(args)
 
     world_env = os.environ.get("WORLD_SIZE")
     if args.gpus is None:

@@ -205,6 +205,80 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(
   }
 }
 
+// The bf16 path of the grouped GEMM on the matrix cores (K a multiple of 32):
+// v_mfma_f32_16x16x32_bf16 with the expert's weight rows as the A operand and
+// the (gathered) token rows as B, both fragments loaded straight from global
+// memory as one 16-byte load per lane (weights are [n][k] and rows [m][k], so a
+// lane's 8 k-values are contiguous). A workgroup owns 64 token rows x 64
+// features of one expert segment; each of its 4 waves takes 16 features (and
+// the 16 matching up-rows for SwiGLU) against all 64 rows, so the row fragments
+// are shared through L1. An accumulator lane holds 4 consecutive features of
+// one token row. Per output element the sum over K has a fixed order.
+template <int SWIGLU>
+__global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wt, const int* __restrict__ plan, int P,
+    int E, int top, int K, int N, bf16_t* __restrict__ out) {
+  const int* offsets = plan;
+  const int* perm = plan + E + 2;
+  int tile = blockIdx.x, e = 0, r0 = 0, r1 = 0;
+  for (; e < E; ++e) {
+    const int s0 = offsets[e], s1 = offsets[e + 1];
+    const int nt = (s1 - s0 + GG_T - 1) / GG_T;
+    if (tile < nt) { r0 = s0 + tile * GG_T; r1 = min(s1, r0 + GG_T); break; }
+    tile -= nt;
+  }
+  if (e == E) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int nb = blockIdx.y * GG_T + wave * 16;         // this wave's 16 features
+  if (nb >= N) return;
+  const int wrows = SWIGLU ? 2 * N : N;
+  const bf16_t* We = Wt + (size_t)e * wrows * K;
+  const int nrow = min(nb + fr, N - 1);                 // clamped: loads stay in range
+  const bf16_t* wg = We + (size_t)nrow * K + fq * 8;
+  const bf16_t* wu = SWIGLU ? We + (size_t)(N + nrow) * K + fq * 8 : nullptr;
+  const bf16_t* arow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = min(r0 + 16 * j + fr, r1 - 1);
+    const size_t src = SWIGLU ? (size_t)(perm[r] / top) : (size_t)r;
+    arow[j] = A + src * K + fq * 8;
+  }
+  float4v acc[4], accu[SWIGLU ? 4 : 1];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (SWIGLU) accu[j] = float4v{0.f, 0.f, 0.f, 0.f};
+  }
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(wg + k0);
+    bf16x8 au;
+    if (SWIGLU) au = *reinterpret_cast<const bf16x8*>(wu + k0);
+    bf16x8 b[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8*>(arow[j] + k0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[j], 0, 0, 0);
+      if (SWIGLU) accu[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au, b[j], accu[j], 0, 0, 0);
+    }
+  }
+  // acc[j][i]: feature nb + 4 fq + i of token row r0 + 16 j + fr
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = r0 + 16 * j + fr;
+    if (r >= r1) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = nb + 4 * fq + i;
+      if (n < N) {
+        const float v = SWIGLU ? silu_f(acc[j][i]) * accu[j][i] : acc[j][i];
+        out[(size_t)r * N + n] = f2bf(v);
+      }
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const T* __restrict__ h, const T* __restrict__ y, const int* __restrict__ idx,
@@ -265,6 +339,15 @@ extern "C" int loqa_moe_grouped_gemm(const void* A, int dt, const void* W, const
                                      hipStream_t st) {
   if (P <= 0) return 0;
   const dim3 grid((P + GG_T - 1) / GG_T + E, (N + GG_T - 1) / GG_T);
+  if (dt == 0 && K >= 32 && K % 32 == 0) {
+    if (swiglu)
+      hipLaunchKernelGGL(moe_grouped_gemm_mfma_kernel<1>, grid, dim3(256), 0, st, (const bf16_t*)A,
+                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
+    else
+      hipLaunchKernelGGL(moe_grouped_gemm_mfma_kernel<0>, grid, dim3(256), 0, st, (const bf16_t*)A,
+                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
+    return (int)hipGetLastError();
+  }
 #define GO(TT, SW)                                                                              \
   hipLaunchKernelGGL((moe_grouped_gemm_kernel<TT, SW>), grid, dim3(256), 0, st, (const TT*)A,   \
                      (const TT*)W, (const int*)plan, P, E, top, K, N, (TT*)out)

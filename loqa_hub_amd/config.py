@@ -221,16 +221,19 @@ class GPUConfig:
     def llm_config(self):
         """The intent model's shape: the checkpoint's own config.json when it
         has one (any Llama-family checkpoint), else the named ``HUB_LLM_MODEL``."""
-        from .models.configs import checkpoint_config, llama_config, llama_config_from_hf
+        from .models.configs import checkpoint_config, llama_config
+        from .models.registry import lm_config_from_json
         d = checkpoint_config(self.llm_checkpoint)
-        return llama_config_from_hf(d, self.llm_model) if d else llama_config(self.llm_model)
+        # the checkpoint's config.json picks the model family (models/registry.py)
+        return lm_config_from_json(d, self.llm_model) if d else llama_config(self.llm_model)
 
     def tp_fallback_config(self):
         """Shape of the TP failover engine: its checkpoint's config.json, else
         ``HUB_TP_FALLBACK_MODEL``."""
-        from .models.configs import checkpoint_config, llama_config, llama_config_from_hf
+        from .models.configs import checkpoint_config, llama_config
+        from .models.registry import lm_config_from_json
         d = checkpoint_config(self.tp_fallback_checkpoint)
-        return llama_config_from_hf(d, self.tp_fallback_model) if d else \
+        return lm_config_from_json(d, self.tp_fallback_model) if d else \
             llama_config(self.tp_fallback_model)
 
     def stt_config(self):

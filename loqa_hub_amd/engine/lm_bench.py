@@ -1,0 +1,133 @@
+"""Prefill and decode throughput of the language-model families through the
+engine's step function, at layer sizes that resemble real models (random
+weights, synthetic tokens): ``python bench.py --lm-bench``.
+
+For each size a Pipizen stack (latent attention / lightning mixers, dense and
+mixture-of-experts feed-forwards) runs beside a Llama stack of the same width,
+depth, head count and feed-forward width - the framework's closest existing
+decoder. Measured per family:
+
+* prefill: one prompt of ``P`` tokens through ``LLMEngine.step_logits``;
+* decode: ``B`` sequences at context ``P`` advancing one token per step
+  (Llama: the fused decode step the scheduler replays; Pipizen: its step
+  function on a [B]-row batch).
+
+One JSON line per (size, family); nothing here touches the default workload.
+"""
+from __future__ import annotations
+
+import json
+import time
+
+import numpy as np
+import torch
+
+from ..models.configs import (FeedForwardConfig, HybridLayerConfig, LatentAttnConfig, LightningConfig,
+                              LlamaConfig, PipizenConfig, RotaryConfig)
+
+SIZES = {
+    # name: (width, layers, heads, head_dim, rot_dim, kv_rank, ff, experts, expert_ff, top)
+    "1b": (2048, 4, 16, 128, 64, 512, 5632, 16, 1408, 4),
+    "7b": (4096, 4, 32, 128, 64, 512, 11008, 32, 1408, 6),
+    "tiny": (64, 4, 2, 16, 8, 24, 96, 4, 32, 2),       # CPU plumbing run
+}
+
+
+def pipizen_stack(name: str, vocab: int = 32000) -> PipizenConfig:
+    d, n, H, D, Dr, R, ff, E, eff, top = SIZES[name]
+    rot = RotaryConfig(Dr, 10000.0, (8.0, 2048.0, 32.0, 1.0))
+    layers = []
+    for i in range(n):
+        if i % 2 == 0:
+            mixer = LatentAttnConfig(H, D, Dr, D, R, (D + Dr) ** -0.5, rot,
+                                     None if i % 4 == 0 else i - 2)
+            kind = "latent_attention"
+        else:
+            mixer = LightningConfig(H, D, D, tuple(0.9 + 0.099 * h / max(1, H - 1) for h in range(H)))
+            kind = "lightning"
+        mlp = FeedForwardConfig("dense", ff) if i % 2 == 0 else \
+            FeedForwardConfig("moe", eff, E, 0, top, 4, 2, eff)
+        layers.append(HybridLayerConfig(kind, mixer, mlp))
+    return PipizenConfig(f"pipizen-{name}", vocab, d, 1e-6, tuple(layers))
+
+
+def llama_stack(name: str, vocab: int = 32000) -> LlamaConfig:
+    d, n, H, D, _, _, ff, _, _, _ = SIZES[name]
+    return LlamaConfig(f"llama-{name}-stack", d, n, H, max(1, H // 4), D, ff, vocab,
+                       rope_theta=10000.0, max_positions=8192)
+
+
+def _sync(dev):
+    if dev.type == "cuda":
+        torch.cuda.synchronize(dev)
+
+
+def _time(fn, dev, reps: int) -> float:
+    fn()
+    _sync(dev)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    _sync(dev)
+    return (time.perf_counter() - t0) / reps
+
+
+def bench_family(cfg, dev, *, prompt: int, batch: int, steps: int, seed: int = 0) -> dict:
+    from .llm_engine import LLMEngine
+    cap = -(-(prompt + steps + 8) // 64) * 64
+    eng = LLMEngine(cfg, dev, seed=seed, max_seqs=batch, max_seq_len=cap, block_size=16,
+                    num_blocks=batch * cap // 16 + 8, use_graphs=False)
+    g = torch.Generator().manual_seed(seed)
+    toks = torch.randint(0, cfg.vocab_size, (batch, prompt), generator=g).tolist()
+    out = {"family": eng.family.name, "model": cfg.name, "prompt": prompt, "batch": batch}
+    with torch.inference_mode():
+        # prefill: each sequence's prompt as one pass (the first is the warm-up)
+        seqs, times = [], []
+        for b in range(batch):
+            s = eng.open_sequence()
+            _sync(eng.device)
+            t0 = time.perf_counter()
+            eng.step_logits([s], [toks[b]], [[prompt - 1]])
+            _sync(eng.device)
+            times.append(time.perf_counter() - t0)
+            seqs.append(s)
+        pre = float(np.median(times[1:])) if batch > 1 else times[0]
+        out["prefill_ms"] = pre * 1e3
+        out["prefill_tok_s"] = prompt / pre
+
+        # decode: all sequences advance one token per step
+        def step():
+            if eng.hybrid:
+                eng.step_logits(seqs, [[1]] * batch, [[0]] * batch)
+                return
+            from .. import ops
+            max_q, max_ctx, host = eng._meta(seqs, [[1]] * batch, True, batch, ops.mpad_for(batch))
+            host["mask_rows"] = np.zeros(batch, np.int32)
+            d = eng._to_device(host)
+            eng._forward_sample(eng._build_meta(d, max_q, max_ctx, True), d["mask_rows"])
+        dt = _time(step, eng.device, steps)
+        out["decode_ms"] = dt * 1e3
+        out["decode_tok_s"] = batch / dt
+    for s in seqs:
+        eng.close_sequence(s)
+    return out
+
+
+def run(args) -> int:
+    dev = torch.device("cuda", 0) if torch.cuda.is_available() and not args.cpu_smoke \
+        else torch.device("cpu")
+    sizes = [s for s in args.lm_sizes.split(",") if s]
+    for name in sizes:
+        for cfg in (pipizen_stack(name), llama_stack(name)):
+            if dev.type == "cpu":      # plumbing run: tiny stacks
+                prompt, batch, steps = 48, 2, 2
+            else:
+                prompt, batch, steps = args.lm_prompt, args.lm_batch, args.lm_steps
+            r = bench_family(cfg, dev, prompt=prompt, batch=batch, steps=steps, seed=args.seed)
+            r["size"] = name
+            r["dtype"] = "bf16"
+            r["data"] = "synthetic"
+            print(json.dumps(r), flush=True)
+            if dev.type == "cuda":
+                torch.cuda.empty_cache()
+    return 0

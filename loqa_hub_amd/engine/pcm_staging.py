@@ -264,7 +264,15 @@ def host_register(addr: int, nbytes: int) -> bool:
     hip = hip_runtime()
     hip.hipHostRegister.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint]
     hip.hipHostRegister.restype = ctypes.c_int
-    return hip.hipHostRegister(ctypes.c_void_p(addr), ctypes.c_size_t(nbytes), 0) == 0
+    ok = hip.hipHostRegister(ctypes.c_void_p(addr), ctypes.c_size_t(nbytes), 0) == 0
+    if not ok:
+        # some machines refuse to pin memory that already exists; the refusal
+        # stays behind as the runtime's last error and would be reported by the
+        # next, unrelated GPU call: take it off here (callers fall back to
+        # staging copies)
+        hip.hipGetLastError.restype = ctypes.c_int
+        hip.hipGetLastError()
+    return ok
 
 
 def host_unregister(addr: int) -> None:

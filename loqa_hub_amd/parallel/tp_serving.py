@@ -68,8 +68,8 @@ def build_tp_llm(lcfg, info: DistInfo, *, seed: int = 0, max_seqs: int = 64,
     tp = TPGroup.create(info.rank, info.world, dist.group.WORLD, device=info.device)
     weights = None
     if checkpoint:
-        from ..models import loader
-        weights = loader.load_llama(lcfg, checkpoint, info.device, tp=tp)
+        from ..models.registry import load_lm_weights
+        weights = load_lm_weights(lcfg, checkpoint, info.device, tp=tp, max_positions=max_seq_len)
     eng = LLMEngine(lcfg, info.device, seed=seed, max_seqs=max_seqs, max_seq_len=max_seq_len,
                     block_size=block_size, tp=tp, use_graphs=use_graphs, weights=weights,
                     compact=compact, tokenizer=tokenizer)
@@ -165,8 +165,9 @@ class TPFailover:
                 weights, tok = None, self.tokenizer
                 if self.checkpoint:
                     from ..engine.tokenizer import find_tokenizer, load_tokenizer
-                    from ..models import loader
-                    weights = loader.load_llama(self.lcfg, self.checkpoint, self.device)
+                    from ..models.registry import load_lm_weights
+                    weights = load_lm_weights(self.lcfg, self.checkpoint, self.device,
+                                              max_positions=self.kw.get("max_seq_len", 1024))
                     if tok is None and find_tokenizer(self.checkpoint):
                         tok = load_tokenizer(self.checkpoint, self.lcfg.vocab_size)
                 eng = LLMEngine(self.lcfg, self.device, weights=weights, tokenizer=tok, **self.kw)

@@ -108,8 +108,9 @@ def build_gpu_processor(cfg: Config, nats, device: str = "cuda:0", tts=None, *, 
     if g.stt_checkpoint or (g.llm_checkpoint and llm is None):
         from .models import loader
         sw = loader.load_whisper(scfg, g.stt_checkpoint, device) if g.stt_checkpoint else None
-        lw = loader.load_llama(lcfg, g.llm_checkpoint, device) if (g.llm_checkpoint and llm is None) \
-            else None
+        from .models.registry import load_lm_weights
+        lw = load_lm_weights(lcfg, g.llm_checkpoint, device, max_positions=g.max_seq_len) \
+            if (g.llm_checkpoint and llm is None) else None
     stt = STTEngine(scfg, device, seed=g.seed, max_batch=g.max_batch, use_graphs=g.use_graphs,
                     weights=sw, tokenizer=g.tokenizer("stt", scfg.vocab_size),
                     language=cfg.stt.language)
