@@ -7,31 +7,37 @@
 //
 // lightning_scan_kernel: one workgroup per (sequence, head, 32 value columns).
 // The columns of S evolve independently, so the grid splits Dv freely. A
-// thread holds S[d, e] for one column e and every 8th row d in registers; the
-// step's tokens are staged 16 at a time in LDS (SiLU applied once), the
-// recurrence then runs token by token in f32 in the order of the definition,
-// and the 8 row-partials of o_t are summed in a fixed order. A prompt portion,
-// a single decode token, or any cut of a prompt therefore gives the same bits.
+// thread holds S[d, e] for one column e and a contiguous run of MAXD rows d in
+// registers (8 threads per column). The step's tokens are staged TC at a time
+// in LDS (SiLU applied once, rows zero-padded to 8 MAXD so the recurrence reads
+// them as float4); the raw values of the next TC tokens are already in flight
+// in registers while the current ones are processed. The recurrence runs token
+// by token in f32 in the order of the definition; the 8 row-partials of o_t
+// are summed in a fixed order (pairs inside a wave, then the 4 waves). A prompt
+// portion, a single decode token, or any cut of a prompt gives the same bits.
 #include "seqmix.h"
 
 #define LS_EC 32        // value columns per workgroup
 #define LS_DP 8         // row partitions (threads per column)
-#define LS_TC 16        // tokens staged per round
 
-template <typename T, int MAXD>   // D <= LS_DP * MAXD
+template <typename T, int MAXD, int TC>   // D <= LS_DP * MAXD
 __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
     const T* __restrict__ qkv, long ld, int H, int D, int Dv, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q,
     const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ o) {
-  extern __shared__ float lds[];
-  float* qs = lds;                         // [TC][D]
-  float* ks = qs + LS_TC * D;              // [TC][D]
-  float* vs = ks + LS_TC * D;              // [TC][EC]
-  float* red = vs + LS_TC * LS_EC;         // [TC][DP][EC]
+  constexpr int DPAD = LS_DP * MAXD;            // padded row length in LDS
+  constexpr int NPT = TC * DPAD / 256;          // staged q (and k) values per thread
+  constexpr int NVT = TC * LS_EC / 256;         // staged v values per thread
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* qs = lds;                         // [TC][DPAD]
+  float* ks = qs + TC * DPAD;              // [TC][DPAD]
+  float* vs = ks + TC * DPAD;              // [TC][EC]
+  float* red = vs + TC * LS_EC;            // [TC][4 waves][EC]
   const int b = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * LS_EC;
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
   if (q1 <= q0) return;
-  const int e = threadIdx.x % LS_EC, dp = threadIdx.x / LS_EC;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e = tid % LS_EC, dp = tid / LS_EC;
   const bool col = e0 + e < Dv;
   const float lam = decay[h];
   float* Sg = state + (((size_t)state_slots[b] * H + h) * D) * Dv + e0 + e;
@@ -39,54 +45,70 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
   float S[MAXD];
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) {
-    const int d = dp + LS_DP * i;
+    const int d = dp * MAXD + i;
     S[i] = (!fresh && col && d < D) ? Sg[(size_t)d * Dv] : 0.f;
   }
   const size_t qoff = (size_t)h * D, koff = (size_t)H * D + (size_t)h * D;
   const size_t voff = 2 * (size_t)H * D + (size_t)h * Dv + e0;
-  for (int t0 = q0; t0 < q1; t0 += LS_TC) {
-    const int nt = min(LS_TC, q1 - t0);
-    __syncthreads();
-    for (int i = threadIdx.x; i < nt * D; i += blockDim.x) {
-      const int tt = i / D, d = i - tt * D;
-      const T* row = qkv + (size_t)(t0 + tt) * ld;
-      qs[i] = silu_f(Act<T>::ld(row + qoff + d));
-      ks[i] = silu_f(Act<T>::ld(row + koff + d));
+  float rq[NPT], rk[NPT], rv[NVT];
+  auto fetch = [&](int t0) {               // raw projections of tokens t0 .. t0 + TC
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+      const int i = tid + 256 * j, tt = i / DPAD, d = i % DPAD;
+      const bool ok = t0 + tt < q1 && d < D;
+      const T* row = qkv + (size_t)(ok ? t0 + tt : q0) * ld;
+      rq[j] = ok ? Act<T>::ld(row + qoff + d) : 0.f;
+      rk[j] = ok ? Act<T>::ld(row + koff + d) : 0.f;
     }
-    for (int i = threadIdx.x; i < nt * LS_EC; i += blockDim.x) {
-      const int tt = i / LS_EC, c = i - tt * LS_EC;
-      vs[i] = e0 + c < Dv ? silu_f(Act<T>::ld(qkv + (size_t)(t0 + tt) * ld + voff + c)) : 0.f;
+#pragma unroll
+    for (int j = 0; j < NVT; ++j) {
+      const int i = tid + 256 * j, tt = i / LS_EC, c = i % LS_EC;
+      const bool ok = t0 + tt < q1 && e0 + c < Dv;
+      rv[j] = ok ? Act<T>::ld(qkv + (size_t)(t0 + tt) * ld + voff + c) : 0.f;
     }
+  };
+  fetch(q0);
+  for (int t0 = q0; t0 < q1; t0 += TC) {
+    const int nt = min(TC, q1 - t0);
+    __syncthreads();                       // the previous round's LDS is consumed
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+      qs[tid + 256 * j] = silu_f(rq[j]);   // silu(0) = 0 keeps the padding zero
+      ks[tid + 256 * j] = silu_f(rk[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < NVT; ++j) vs[tid + 256 * j] = silu_f(rv[j]);
     __syncthreads();
+    if (t0 + TC < q1) fetch(t0 + TC);      // in flight during the recurrence below
     for (int tt = 0; tt < nt; ++tt) {
       const float v = vs[tt * LS_EC + e];
-      const float* kq = ks + tt * D;
-      const float* qq = qs + tt * D;
+      const float4* k4 = reinterpret_cast<const float4*>(ks + tt * DPAD + dp * MAXD);
+      const float4* q4 = reinterpret_cast<const float4*>(qs + tt * DPAD + dp * MAXD);
       float part = 0.f;
 #pragma unroll
-      for (int i = 0; i < MAXD; ++i) {
-        const int d = dp + LS_DP * i;
-        if (d < D) {
-          S[i] = lam * S[i] + kq[d] * v;
-          part += S[i] * qq[d];
-        }
+      for (int i = 0; i < MAXD / 4; ++i) {
+        const float4 kk = k4[i], qq = q4[i];
+        S[4 * i] = lam * S[4 * i] + kk.x * v;         part += S[4 * i] * qq.x;
+        S[4 * i + 1] = lam * S[4 * i + 1] + kk.y * v; part += S[4 * i + 1] * qq.y;
+        S[4 * i + 2] = lam * S[4 * i + 2] + kk.z * v; part += S[4 * i + 2] * qq.z;
+        S[4 * i + 3] = lam * S[4 * i + 3] + kk.w * v; part += S[4 * i + 3] * qq.w;
       }
-      red[(tt * LS_DP + dp) * LS_EC + e] = part;
+      part += __shfl_xor(part, 32, 64);    // the wave's two row partitions
+      if (lane < 32) red[(tt * 4 + wave) * LS_EC + e] = part;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < nt * LS_EC; i += blockDim.x) {
-      const int tt = i / LS_EC, c = i - tt * LS_EC;
+    for (int i = tid; i < nt * LS_EC; i += 256) {
+      const int tt = i / LS_EC, c = i % LS_EC;
       if (e0 + c < Dv) {
-        float s = 0.f;
-#pragma unroll
-        for (int k = 0; k < LS_DP; ++k) s += red[(tt * LS_DP + k) * LS_EC + c];
-        o[(size_t)(t0 + tt) * H * Dv + (size_t)h * Dv + e0 + c] = s;
+        const float* r = red + tt * 4 * LS_EC + c;
+        o[(size_t)(t0 + tt) * H * Dv + (size_t)h * Dv + e0 + c] =
+            ((r[0] + r[LS_EC]) + r[2 * LS_EC]) + r[3 * LS_EC];
       }
     }
   }
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) {
-    const int d = dp + LS_DP * i;
+    const int d = dp * MAXD + i;
     if (col && d < D) Sg[(size_t)d * Dv] = S[i];
   }
 }
@@ -117,14 +139,14 @@ extern "C" int loqa_lightning_scan(const void* qkv, int dt, long ld, int H, int 
   if (D > LS_DP * 32 || D <= 0 || Dv <= 0) return (int)hipErrorInvalidValue;
   (void)nslots;
   const dim3 grid(B, H, (Dv + LS_EC - 1) / LS_EC), block(LS_EC * LS_DP);
-  const size_t smem = (size_t)(2 * LS_TC * D + LS_TC * LS_EC + LS_TC * LS_DP * LS_EC) * 4;
-#define GO(TT, MD)                                                                             \
-  hipLaunchKernelGGL((lightning_scan_kernel<TT, MD>), grid, block, smem, st, (const TT*)qkv, ld, H, \
-                     D, Dv, (float*)state, (const int*)state_slots, (const int*)cu_q,          \
-                     (const int*)positions, (const float*)decay, (float*)o)
+#define GO(TT, MD, TCC)                                                                          \
+  hipLaunchKernelGGL((lightning_scan_kernel<TT, MD, TCC>), grid, block,                          \
+                     (size_t)(2 * TCC * LS_DP * MD + TCC * LS_EC + TCC * 4 * LS_EC) * 4, st,     \
+                     (const TT*)qkv, ld, H, D, Dv, (float*)state, (const int*)state_slots,       \
+                     (const int*)cu_q, (const int*)positions, (const float*)decay, (float*)o)
   const int md = D <= 64 ? 8 : (D <= 128 ? 16 : 32);
-  if (dt == 0) { if (md == 8) GO(bf16_t, 8); else if (md == 16) GO(bf16_t, 16); else GO(bf16_t, 32); }
-  else { if (md == 8) GO(float, 8); else if (md == 16) GO(float, 16); else GO(float, 32); }
+  if (dt == 0) { if (md == 8) GO(bf16_t, 8, 32); else if (md == 16) GO(bf16_t, 16, 32); else GO(bf16_t, 32, 16); }
+  else { if (md == 8) GO(float, 8, 32); else if (md == 16) GO(float, 16, 32); else GO(float, 32, 16); }
 #undef GO
   return (int)hipGetLastError();
 }

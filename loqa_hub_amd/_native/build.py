@@ -82,9 +82,10 @@ def _build_lib(name: str, sources: list[str], headers: list[str], flags: list[st
 
 
 # The sequence-mixer kernels of the hybrid decoders are a library of their own:
-# a checkout that only replays or serves such a model compiles these four files
+# a checkout that only replays or serves such a model compiles these few files
 # (seconds) and not the whole kernel set (minutes).
-SEQMIX_SOURCES = ("norm_dyt.hip", "attn_latent.hip", "lightning.hip", "moe.hip")
+SEQMIX_SOURCES = ("norm_dyt.hip", "attn_latent.hip", "attn_latent_prefill.hip", "lightning.hip",
+                  "moe.hip")
 
 # hipcc may not form packed-f32 VALU instructions from scalar float code
 NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

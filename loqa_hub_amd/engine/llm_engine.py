@@ -255,11 +255,19 @@ class LLMEngine:
         if self.hybrid:
             host["state_slots"] = np.asarray(
                 self.kv.state_slots([r.seq_id for r in seqs], B_pad), np.int32)
+            # where each sequence's context starts in a gathered key buffer
+            cu_k = np.zeros(B_pad + 1, np.int32)
+            np.cumsum(ctx[:B_pad], out=cu_k[1:])
+            host["cu_k"] = cu_k
+            host["total_k"] = int(cu_k[-1])
         return max_q, max_ctx, host
 
     def _to_device(self, host: dict, dst: dict | None = None) -> dict:
         out = {}
         for k, a in host.items():
+            if not isinstance(a, np.ndarray):      # host-side scalars ride along
+                out[k] = a
+                continue
             t = torch.from_numpy(a)
             if self.is_gpu:
                 t = t.pin_memory()
@@ -319,7 +327,8 @@ class LLMEngine:
         return StepMeta(tokens=dev["tokens"], positions=dev["positions"], slots=dev["slots"],
                         cu_q=dev["cu_q"], ctx_lens=dev["ctx_lens"], block_tables=dev["block_tables"],
                         logit_idx=dev["logit_idx"], max_q=max_q, max_ctx=max_ctx, decode=decode,
-                        state_slots=dev.get("state_slots"))
+                        state_slots=dev.get("state_slots"), cu_k=dev.get("cu_k"),
+                        total_k=dev.get("total_k", 0))
 
     CTX_BUCKET = 256
 

@@ -47,6 +47,10 @@ class StepMeta:
     split: tuple | None = None
     # state slot of each sequence (models with recurrent layers), int32 [B]
     state_slots: torch.Tensor | None = None
+    # start of each sequence's context in a gathered key buffer, int32 [B + 1],
+    # and the buffer's row count (latent attention's prompt path)
+    cu_k: torch.Tensor | None = None
+    total_k: int = 0
 
 
 class TPGroup:

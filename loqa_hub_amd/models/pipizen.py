@@ -70,6 +70,7 @@ class PipizenWeights:
                 H, D, Dr, Dv, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
                 L["wq"] = W(p + "mix.q")
                 assert L["wq"].shape[0] == H * (D + Dr)
+                L["qw"] = D + Dr          # per-head width of the query projection
                 if m.kv_from is None:
                     L["wdkv"] = W(p + "mix.dkv")
                     L["dkv_norm"] = F(p + "mix.dkv.norm")
@@ -81,6 +82,7 @@ class PipizenWeights:
                 L["sink"] = F(p + "mix.sink") if (p + "mix.sink") in sd else None
                 L["wo"] = W(p + "mix.o")
                 L["cos_sin"] = self._table(m.rot)
+                self._prompt_layout(L, m)
             else:
                 L["wqkvg"] = torch.cat([W(p + "mix.q"), W(p + "mix.k"), W(p + "mix.v"),
                                         W(p + "mix.g")]).contiguous()
@@ -107,6 +109,31 @@ class PipizenWeights:
                                                     W(p + "mlp.shared.up")]).contiguous()
                         L["s_down"] = W(p + "mlp.shared.down")
             self.layers.append(L)
+
+    def _prompt_layout(self, L: dict, m) -> None:
+        """Padded per-head copies for the matrix-core prompt kernel (bf16): the
+        query projection with DKp rows per head, W_uk / W_uv producing [H, DKp]
+        keys and [H, DVp] values from a latent row, and W_o with DVp columns per
+        head. Sizes that the kernel is built for are used as they are."""
+        H, D, Dr, Dv, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
+        sizes = seqmix.prefill_head_sizes(D + Dr, Dv) if self.dtype == torch.bfloat16 else None
+        if sizes is None or self.device.type != "cuda":
+            return
+        DKp, DVp = sizes
+        dev, dt = self.device, self.dtype
+
+        def pad_rows(w, per, to):       # [H * per, n] -> [H * to, n], zero rows after each head
+            if per == to:
+                return w
+            out = torch.zeros(H, to, w.shape[1], dtype=dt, device=dev)
+            out[:, :per] = w.view(H, per, -1)
+            return out.view(H * to, -1).contiguous()
+        L["wq"], L["qw"] = pad_rows(L["wq"], D + Dr, DKp), DKp
+        L["wuk_p"] = pad_rows(L["wuk"].reshape(H * D, R), D, DKp)
+        L["wuv_p"] = pad_rows(L["wuv_t"].transpose(1, 2).reshape(H * Dv, R), Dv, DVp)
+        L["wo_p"] = L["wo"] if DVp == Dv else \
+            pad_rows(L["wo"].t().contiguous(), Dv, DVp).t().contiguous()
+        L["prompt_sizes"] = (DKp, DVp)
 
     def _table(self, rot) -> torch.Tensor:
         key = (rot.dims, rot.base, rot.yarn)
@@ -218,6 +245,10 @@ class PipizenModel:
     reading and extending the paged latent cache and the state slots."""
 
     hybrid = True
+    # a step whose longest feed has at least this many tokens takes the
+    # matrix-core prompt path of latent attention (bf16 on the GPU); shorter
+    # feeds (decode, short tails) read the latent pages directly
+    prompt_min_q = 32
 
     def __init__(self, w: PipizenWeights):
         self.w, self.cfg = w, w.cfg
@@ -271,9 +302,22 @@ class PipizenModel:
             z = ops.linear(h, L["wdkv"])
             seqmix.latent_append(z, L["dkv_norm"], self.cfg.norm_eps, meta.positions, L["cos_sin"],
                                  pages, meta.slots, R, m.rot.dims)
-        q = ops.linear(h, L["wq"]).view(T, H, D + Dr)
+        q = ops.linear(h, L["wq"]).view(T, H, L["qw"])
+        if "prompt_sizes" in L and meta.max_q >= self.prompt_min_q and meta.cu_k is not None:
+            # prompt pass: per-head keys / values from the gathered latents, then
+            # flash attention on the matrix cores
+            DKp, DVp = L["prompt_sizes"]
+            cl, kr = seqmix.latent_gather(pages, meta.block_tables, meta.cu_k, meta.total_k,
+                                          meta.max_ctx, R)
+            k = ops.linear(cl, L["wuk_p"]).view(-1, H, DKp)
+            seqmix.latent_kfill_(k, kr, D)
+            v = ops.linear(cl, L["wuv_p"]).view(-1, H, DVp)
+            seqmix.rope_pairs_(q, D, m.rot.dims, meta.positions, L["cos_sin"])
+            o = seqmix.latent_prefill(q, k, v, meta.cu_q, meta.cu_k, meta.positions, L["sink"],
+                                      m.scale, meta.max_q)
+            return ops.linear(o, L["wo_p"])
         qa = torch.bmm(q[:, :, :D].transpose(0, 1), L["wuk"])            # [H, T, R]
-        lat = seqmix.latent_attention(qa, q[:, :, D:], pages, meta.cu_q, meta.ctx_lens,
+        lat = seqmix.latent_attention(qa, q[:, :, D:D + Dr], pages, meta.cu_q, meta.ctx_lens,
                                       meta.block_tables, meta.positions, L["cos_sin"], L["sink"],
                                       m.scale, R, m.rot.dims, meta.max_ctx)
         o = torch.bmm(lat, L["wuv_t"])                                    # [H, T, Dv]

@@ -153,6 +153,82 @@ def latent_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Tensor, cu
     return out
 
 
+PREFILL_DK = (64, 128, 192, 256)     # head sizes the matrix-core prompt kernel is built for
+PREFILL_DV = (64, 128)
+
+
+def prefill_head_sizes(dk: int, dv: int) -> tuple[int, int] | None:
+    """The (padded) key and value head sizes of the prompt-pass kernel for a
+    model's sizes, or None when it does not cover them."""
+    a = next((x for x in PREFILL_DK if x >= dk), None)
+    b = next((x for x in PREFILL_DV if x >= dv), None)
+    return None if a is None or b is None else (a, b)
+
+
+def latent_gather(cache: torch.Tensor, block_tables: torch.Tensor, cu_k: torch.Tensor,
+                  total_k: int, max_ctx: int, R: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Every sequence's cached rows in position order, as contiguous latents
+    [total_k, R] and rotary key parts [total_k, Dr] (bf16, GPU)."""
+    assert cache.is_cuda and cache.dtype == torch.bfloat16 and cache.is_contiguous()
+    _i32c(block_tables, "block_tables"); _i32c(cu_k, "cu_k")
+    B, Dr = block_tables.shape[0], cache.shape[2] - R
+    assert cu_k.numel() == B + 1
+    cl = torch.empty(total_k, R, dtype=cache.dtype, device=cache.device)
+    kr = torch.empty(total_k, Dr, dtype=cache.dtype, device=cache.device)
+    check(kernels().loqa_latent_gather(ptr(cache), cache.shape[1], ptr(block_tables),
+                                       block_tables.shape[1], ptr(cu_k), B, int(max_ctx), R, Dr,
+                                       ptr(cl), ptr(kr), stream_ptr(cache)), "latent_gather")
+    return cl, kr
+
+
+def latent_kfill_(k: torch.Tensor, kr: torch.Tensor, D: int) -> None:
+    """k [L, H, DK] (bf16): every head's entries D .. D + Dr take kr [L, Dr]."""
+    L, H, DK = k.shape
+    Dr = kr.shape[1]
+    assert k.is_contiguous() and kr.is_contiguous() and kr.shape[0] == L and D + Dr <= DK
+    assert k.dtype == kr.dtype == torch.bfloat16
+    check(kernels().loqa_latent_kfill(ptr(k), ptr(kr), L, H, DK, D, Dr, stream_ptr(k)),
+          "latent_kfill")
+
+
+def rope_pairs_(x: torch.Tensor, off: int, dims: int, positions: torch.Tensor,
+                cos_sin: torch.Tensor) -> None:
+    """Rotate in place the interleaved pairs x[t, h, off : off + dims] (bf16)."""
+    T, H, _ = x.shape
+    assert x.dtype == torch.bfloat16 and x.stride(2) == 1 and off + dims <= x.shape[2]
+    _i32c(positions, "positions"); _f32c(cos_sin, "cos_sin")
+    assert cos_sin.shape[1] * 2 == dims and positions.numel() >= T
+    check(kernels().loqa_rope_pairs(ptr(x), x.stride(0), x.stride(1), T, H, off, dims,
+                                    ptr(positions), ptr(cos_sin), cos_sin.shape[0], stream_ptr(x)),
+          "rope_pairs")
+
+
+def latent_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_q: torch.Tensor,
+                   cu_k: torch.Tensor, positions: torch.Tensor, sink: torch.Tensor | None,
+                   scale: float, max_q: int) -> torch.Tensor:
+    """Causal flash attention of a prompt pass on the matrix cores: q [T, H, DK]
+    (rotated), k [L, H, DK], v [L, H, DV] per-head keys / values of the
+    gathered contexts (``cu_k``), a query at absolute position p sees keys
+    0 .. p of its sequence; ``sink`` [H] joins the softmax denominator.
+    Returns [T, H * DV] (bf16)."""
+    T, H, DK = q.shape
+    DV = v.shape[2]
+    assert q.is_cuda and q.dtype == k.dtype == v.dtype == torch.bfloat16
+    assert q.stride(2) == 1 and q.stride(1) == DK and k.is_contiguous() and v.is_contiguous()
+    assert k.shape[1:] == (H, DK) and v.shape[:2] == k.shape[:2]
+    assert DK in PREFILL_DK and DV in PREFILL_DV
+    _i32c(cu_q, "cu_q"); _i32c(cu_k, "cu_k"); _i32c(positions, "positions")
+    B = cu_q.numel() - 1
+    assert cu_k.numel() == B + 1
+    if sink is not None:
+        _f32c(sink, "sink")
+    o = torch.empty(T, H * DV, dtype=q.dtype, device=q.device)
+    check(kernels().loqa_latent_prefill(ptr(q), q.stride(0), ptr(k), ptr(v), ptr(o), ptr(cu_q),
+                                        ptr(cu_k), ptr(positions), ptr(sink), float(scale), B, H,
+                                        int(max_q), DK, DV, stream_ptr(q)), "latent_prefill")
+    return o
+
+
 def lightning_scan(qkv: torch.Tensor, H: int, D: int, Dv: int, state: torch.Tensor,
                    state_slots: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor,
                    decay: torch.Tensor) -> torch.Tensor:

@@ -372,3 +372,61 @@ def test_trace_replay_program(tmp_path, full_model):
     assert not (out / "1.f32").exists()
     assert rel_err(g0, wa[[0, 10]]) < TOL[torch.float32]
     assert rel_err(g2, torch.stack([wa[19], wb[8]])) < TOL[torch.float32]
+
+
+# ------------------------------------------- matrix-core paths (bf16, GPU only)
+@pytest.mark.gpu
+def test_prompt_path_matches_folded_attention(full_model):
+    """bf16 on the GPU: prompt passes run latent attention on per-head keys and
+    values (head sizes padded to the kernel's) while short feeds read the latent
+    pages directly; both agree with each other within 16-bit rounding, for
+    whole prompts, portions on top of a cached context and an unequal batch."""
+    from loqa_hub_amd.models.pipizen import PipizenModel
+    cfg = O.make_config([(O.latent(heads=3, dim=16, rot_dim=8, vdim=12, kv_rank=32), None),
+                         (O.latent(heads=3, dim=16, rot_dim=8, vdim=12, kv_rank=32, kv_from=0),
+                          O.dense(64)),
+                         (O.latent(heads=2, dim=96, rot_dim=32, vdim=128, kv_rank=64, scaling=False),
+                          None)], width=64, vocab=100)
+    sd = O.make_weights(cfg, 5)
+    a, b = tokens(150, 100, 1), tokens(40, 100, 2)
+    want_a, want_b = O.forward(cfg, sd, a), O.forward(cfg, sd, b)
+    outs = {}
+    for name, min_q in (("prompt", 1), ("folded", 10 ** 9)):
+        eng = engine(cfg, sd, "cuda", torch.bfloat16, max_tokens=256)
+        assert "prompt_sizes" in eng.weights.layers[0]
+        eng.model.prompt_min_q = min_q
+        sa, sb = eng.open_sequence(), eng.open_sequence()
+        got_a = [eng.step_logits([sa], [a[:70]], [list(range(70))])]
+        o = eng.step_logits([sa, sb], [a[70:133], b[:39]], [list(range(63)), list(range(39))])
+        got_a.append(o[:63])
+        got_b = [o[63:]]
+        o = eng.step_logits([sa, sb], [a[133:], b[39:]], [list(range(17)), [0]])
+        got_a.append(o[:17])
+        got_b.append(o[17:])
+        outs[name] = (torch.cat(got_a), torch.cat(got_b))
+    assert PipizenModel.prompt_min_q > 1
+    for i, want in enumerate((want_a, want_b)):
+        assert rel_err(outs["prompt"][i], outs["folded"][i].double().cpu(), 0.9) < 0.05
+        assert rel_err(outs["prompt"][i], want, 0.5) < 0.06
+        assert rel_err(outs["folded"][i], want, 0.5) < 0.06
+
+
+@pytest.mark.gpu
+def test_grouped_expert_gemm_matrix_cores():
+    """The bf16 grouped expert GEMMs on the matrix cores (K a multiple of 32)
+    against the f32 reference: unequal expert loads, an empty expert, identity
+    experts, segments that do not fill a tile."""
+    from loqa_hub_amd.ops import reference as ref
+    from loqa_hub_amd.ops import seqmix
+    g = torch.Generator().manual_seed(3)
+    T, d, F, E, top = 333, 96, 64, 7, 3
+    h = torch.randn(T, d, generator=g).to(torch.bfloat16)
+    wgu = (torch.randn(E, 2 * F, d, generator=g) / d ** 0.5).to(torch.bfloat16)
+    wd = (torch.randn(E, d, F, generator=g) / F ** 0.5).to(torch.bfloat16)
+    idx = torch.randint(0, E + 2, (T, top), generator=g).to(torch.int32)
+    idx[idx == 4] = 5                                      # expert 4 gets nothing
+    wt = torch.rand(T, top, generator=g)
+    want = ref.moe_experts(h.float(), idx, wt, wgu.float(), wd.float(), torch.float32)
+    got = seqmix.moe_experts(h.cuda(), idx.cuda(), wt.cuda(), wgu.cuda(), wd.cuda()).cpu()
+    err = (got - want).abs().max() / want.abs().max()
+    assert err < 2e-2, float(err)
