@@ -192,6 +192,172 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_attn_kernel(LatAttnParams 
   }
 }
 
+// The same computation for even R and R + Dr (every real configuration), laid
+// out for throughput: the key tile sits in LDS in the activation dtype (twice
+// the keys per tile for bf16), the score of a key is split over two lanes (each
+// half of the wave takes half of the row, read two entries at a time, two
+// independent accumulators), and for P.C a lane owns pairs of output entries.
+#define LAT_MAXP 8      // R <= 128 * LAT_MAXP
+
+template <typename T> struct Pair;
+template <> struct Pair<bf16_t> {
+  static __device__ __forceinline__ float2 ld(const bf16_t* p) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+    return make_float2(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+  }
+};
+template <> struct Pair<float> {
+  static __device__ __forceinline__ float2 ld(const float* p) {
+    return *reinterpret_cast<const float2*>(p);
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(LAT_THREADS) void latent_attn2_kernel(LatAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int W = p.R + p.Dr, Ws = W + 2, KT = p.KT;      // KT <= 32; Ws / 2 odd or even: rows shift banks
+  float* qs = lds;                                      // [4][W] f32, pre-scaled
+  float* ps = qs + LAT_WAVES * W;                       // [4][KT]
+  T* ktile = reinterpret_cast<T*>(ps + LAT_WAVES * KT); // [KT][Ws]
+  const int t = blockIdx.x, split = blockIdx.z;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h_raw = blockIdx.y * LAT_WAVES + wave;
+  const bool live = h_raw < p.H;
+  const int h = live ? h_raw : p.H - 1;
+  T* out = (T*)p.out + ((size_t)h * p.T + t) * p.R;
+  float* wsr = p.num_splits > 1
+      ? p.ws + (((size_t)split * p.T + t) * p.H + h) * (p.R + 2) : nullptr;
+  int nk = 0, b = 0;
+  if (t < p.cu_q[p.B]) {
+    while (b + 1 < p.B && t >= p.cu_q[b + 1]) ++b;
+    nk = min(p.pos[t] + 1, p.ctx[b]);
+  }
+  int k0 = 0, k1 = nk;
+  if (p.num_splits > 1) {
+    const int per = ((nk + p.num_splits - 1) / p.num_splits + KT - 1) / KT * KT;
+    k0 = min(nk, split * per);
+    k1 = min(nk, k0 + per);
+  }
+  {
+    const T* qa = (const T*)p.qa + (size_t)t * p.qa_st + (size_t)h * p.qa_sh;
+    const T* qr = (const T*)p.qr + (size_t)t * p.qr_st + (size_t)h * p.qr_sh;
+    const int pp = min(max(p.pos[t], 0), p.max_pos - 1);
+    const float* csr = p.cs + (size_t)pp * p.dims;
+    for (int i = lane; i < W; i += 64) {
+      float v;
+      if (i < p.R) {
+        v = Act<T>::ld(qa + i);
+      } else {
+        const int j = i - p.R;
+        if (j < p.dims) {
+          const float c = csr[(j >> 1) * 2], s = csr[(j >> 1) * 2 + 1];
+          const float u = Act<T>::ld(qr + (j & ~1)), w = Act<T>::ld(qr + (j | 1));
+          v = (j & 1) ? w * c + u * s : u * c - w * s;
+        } else {
+          v = Act<T>::ld(qr + j);
+        }
+      }
+      qs[wave * W + i] = v * p.scale;
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  float2 acc[LAT_MAXP];
+#pragma unroll
+  for (int i = 0; i < LAT_MAXP; ++i) acc[i] = make_float2(0.f, 0.f);
+  const T* cache = (const T*)p.cache;
+  const int* bt = p.bt + (size_t)b * p.max_blocks;
+  const int key_l = lane & 31, half = lane >> 5;
+  // the two halves of a row, in pairs: [0, hp) and [hp, W / 2)
+  const int npair = W >> 1, hp = (npair + 1) >> 1;
+  const int c_lo = half ? hp : 0, c_hi = half ? npair : hp;
+  for (int kt = k0; kt < k1; kt += KT) {
+    __syncthreads();
+    for (int j = wave; j < KT; j += LAT_WAVES) {
+      const int key = kt + j;
+      uint32_t* dst = reinterpret_cast<uint32_t*>(ktile + (size_t)j * Ws);
+      if (key < k1) {
+        const T* src = cache + ((size_t)bt[key / p.blk] * p.blk + key % p.blk) * W;
+        if (sizeof(T) == 2) {
+          const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src);
+          for (int c = lane; c < npair; c += 64) dst[c] = s32[c];
+        } else {
+          const float* sf = reinterpret_cast<const float*>(src);
+          float* df = reinterpret_cast<float*>(dst);
+          for (int c = lane; c < W; c += 64) df[c] = sf[c];
+        }
+      }
+    }
+    __syncthreads();
+    float s = -INFINITY;
+    const bool has = key_l < KT && kt + key_l < k1;
+    if (has) {
+      const T* kr = ktile + (size_t)key_l * Ws;
+      const float* q = qs + wave * W;
+      float a0 = 0.f, a1 = 0.f;
+      for (int c = c_lo; c < c_hi; ++c) {
+        const float2 kk = Pair<T>::ld(kr + 2 * c);
+        const float2 qq = *reinterpret_cast<const float2*>(q + 2 * c);
+        a0 += qq.x * kk.x;
+        a1 += qq.y * kk.y;
+      }
+      s = a0 + a1;
+    }
+    {
+      const float o = __shfl_xor(s, 32, 64);        // the other half of the row
+      if (has) s += o;
+    }
+    const float mn = fmaxf(m, wave_max(s));
+    const float pj = (has && half == 0) ? expf(s - mn) : 0.f;
+    const float corr = m == -INFINITY ? 0.f : expf(m - mn);
+    l = l * corr + wave_sum(pj);
+    m = mn;
+    if (lane < KT) ps[wave * KT + lane] = pj;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < LAT_MAXP; ++i) { acc[i].x *= corr; acc[i].y *= corr; }
+    const int nj = min(KT, k1 - kt);
+    for (int j = 0; j < nj; ++j) {
+      const float pv = ps[wave * KT + j];
+      const T* cr = ktile + (size_t)j * Ws;
+#pragma unroll
+      for (int i = 0; i < LAT_MAXP; ++i) {
+        const int r = 2 * (lane + 64 * i);
+        if (r < p.R) {
+          const float2 cc = Pair<T>::ld(cr + r);
+          acc[i].x += pv * cc.x;
+          acc[i].y += pv * cc.y;
+        }
+      }
+    }
+  }
+  if (!live) return;
+  if (wsr) {
+    if (lane == 0) { wsr[0] = m; wsr[1] = l; }
+#pragma unroll
+    for (int i = 0; i < LAT_MAXP; ++i) {
+      const int r = 2 * (lane + 64 * i);
+      if (r < p.R) { wsr[2 + r] = acc[i].x; wsr[3 + r] = acc[i].y; }
+    }
+    return;
+  }
+  float M = m, den = l, f = 1.f;
+  if (p.sink) {
+    const float sk = p.sink[h];
+    M = fmaxf(m, sk);
+    f = m == -INFINITY ? 0.f : expf(m - M);
+    den = l * f + expf(sk - M);
+  }
+  const float inv = den > 0.f ? f / den : 0.f;
+#pragma unroll
+  for (int i = 0; i < LAT_MAXP; ++i) {
+    const int r = 2 * (lane + 64 * i);
+    if (r < p.R) {
+      Act<T>::st(out + r, acc[i].x * inv);
+      Act<T>::st(out + r + 1, acc[i].y * inv);
+    }
+  }
+}
+
 // out[h, t] from the key splits' (m, l, acc) partials, merged in split order.
 template <typename T>
 __global__ __launch_bounds__(64) void latent_combine_kernel(
@@ -256,6 +422,28 @@ extern "C" int loqa_latent_attention(
   p.B = B; p.H = H; p.T = T; p.R = R; p.Dr = Dr; p.dims = dims; p.out = out;
   p.num_splits = num_splits < 1 ? 1 : num_splits; p.ws = (float*)ws;
   const int W = R + Dr, Ws = W | 1;
+  if (W % 2 == 0 && R % 2 == 0 && R <= 128 * LAT_MAXP) {
+    const size_t esz = dt == 0 ? 2 : 4;
+    int KT2 = 32;
+    while (KT2 > 4 && (size_t)(LAT_WAVES * W + LAT_WAVES * KT2) * 4 + (size_t)KT2 * (W + 2) * esz > 60 * 1024)
+      KT2 >>= 1;
+    const size_t smem2 = (size_t)(LAT_WAVES * W + LAT_WAVES * KT2) * 4 + (size_t)KT2 * (W + 2) * esz;
+    if (smem2 <= 64 * 1024) {
+      p.KT = KT2;
+      const dim3 grid2(T, (H + LAT_WAVES - 1) / LAT_WAVES, p.num_splits);
+      if (dt == 0) hipLaunchKernelGGL(latent_attn2_kernel<bf16_t>, grid2, dim3(LAT_THREADS), smem2, st, p);
+      else hipLaunchKernelGGL(latent_attn2_kernel<float>, grid2, dim3(LAT_THREADS), smem2, st, p);
+      int rc2 = (int)hipGetLastError();
+      if (rc2 || p.num_splits == 1) return rc2;
+      if (dt == 0)
+        hipLaunchKernelGGL(latent_combine_kernel<bf16_t>, dim3(T, H), dim3(64), 0, st,
+                           (const float*)ws, (const float*)sink, (bf16_t*)out, T, H, R, p.num_splits);
+      else
+        hipLaunchKernelGGL(latent_combine_kernel<float>, dim3(T, H), dim3(64), 0, st,
+                           (const float*)ws, (const float*)sink, (float*)out, T, H, R, p.num_splits);
+      return (int)hipGetLastError();
+    }
+  }
   int KT = 64;
   while (KT > 4 && ((size_t)KT * Ws + LAT_WAVES * W + LAT_WAVES * KT) * 4 > 60 * 1024) KT >>= 1;
   p.KT = KT;

@@ -80,19 +80,24 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
     for (int j = 0; j < NVT; ++j) vs[tid + 256 * j] = silu_f(rv[j]);
     __syncthreads();
     if (t0 + TC < q1) fetch(t0 + TC);      // in flight during the recurrence below
+    // two tokens per trip: the second token's LDS reads and read-out sums are
+    // independent of the first's, so they overlap its latency (only the S
+    // updates chain); four partial sums per token in a fixed order
+#pragma unroll 2
     for (int tt = 0; tt < nt; ++tt) {
       const float v = vs[tt * LS_EC + e];
       const float4* k4 = reinterpret_cast<const float4*>(ks + tt * DPAD + dp * MAXD);
       const float4* q4 = reinterpret_cast<const float4*>(qs + tt * DPAD + dp * MAXD);
-      float part = 0.f;
+      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) {
         const float4 kk = k4[i], qq = q4[i];
-        S[4 * i] = lam * S[4 * i] + kk.x * v;         part += S[4 * i] * qq.x;
-        S[4 * i + 1] = lam * S[4 * i + 1] + kk.y * v; part += S[4 * i + 1] * qq.y;
-        S[4 * i + 2] = lam * S[4 * i + 2] + kk.z * v; part += S[4 * i + 2] * qq.z;
-        S[4 * i + 3] = lam * S[4 * i + 3] + kk.w * v; part += S[4 * i + 3] * qq.w;
+        S[4 * i] = lam * S[4 * i] + kk.x * v;         p0 += S[4 * i] * qq.x;
+        S[4 * i + 1] = lam * S[4 * i + 1] + kk.y * v; p1 += S[4 * i + 1] * qq.y;
+        S[4 * i + 2] = lam * S[4 * i + 2] + kk.z * v; p2 += S[4 * i + 2] * qq.z;
+        S[4 * i + 3] = lam * S[4 * i + 3] + kk.w * v; p3 += S[4 * i + 3] * qq.w;
       }
+      float part = (p0 + p1) + (p2 + p3);
       part += __shfl_xor(part, 32, 64);    // the wave's two row partitions
       if (lane < 32) red[(tt * 4 + wave) * LS_EC + e] = part;
     }
