@@ -279,6 +279,100 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
   }
 }
 
+// Prompt-sized batches (hundreds of rows per expert): 128 token rows x 64
+// features per workgroup, the token rows of a 64-wide K chunk staged once in
+// LDS for the 4 waves (the next chunk's rows already in flight in registers),
+// weights streamed straight from global memory - every weight fragment is
+// loaded once per workgroup and feeds 8 MFMAs, every staged row fragment 2
+// (gate and up). Same fragment layout and summation order as the kernel above.
+#define GG_R2 128
+#define GG_KC 64
+
+template <int SWIGLU>
+__global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wt, const int* __restrict__ plan, int P,
+    int E, int top, int K, int N, bf16_t* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) bf16_t rows[GG_R2][GG_KC + 8];
+  const int* offsets = plan;
+  const int* perm = plan + E + 2;
+  int tile = blockIdx.x, e = 0, r0 = 0, r1 = 0;
+  for (; e < E; ++e) {
+    const int s0 = offsets[e], s1 = offsets[e + 1];
+    const int nt = (s1 - s0 + GG_R2 - 1) / GG_R2;
+    if (tile < nt) { r0 = s0 + tile * GG_R2; r1 = min(s1, r0 + GG_R2); break; }
+    tile -= nt;
+  }
+  if (e == E) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int nb = blockIdx.y * 64 + wave * 16;
+  const bool wave_on = nb < N;                           // idle waves still stage rows
+  const int wrows = SWIGLU ? 2 * N : N;
+  const bf16_t* We = Wt + (size_t)e * wrows * K;
+  const int nrow = min(nb + fr, N - 1);
+  const bf16_t* wg = We + (size_t)nrow * K + fq * 8;
+  const bf16_t* wu = SWIGLU ? We + (size_t)(N + nrow) * K + fq * 8 : nullptr;
+  // staging: thread -> 4 chunks of 8 entries: row = (tid + 256 j) / 8, column chunk = % 8
+  const bf16_t* srow[4];
+  int srr[4], scc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    srr[j] = i >> 3;
+    scc[j] = (i & 7) * 8;
+    const int r = min(r0 + srr[j], r1 - 1);
+    const size_t src = SWIGLU ? (size_t)(perm[r] / top) : (size_t)r;
+    srow[j] = A + src * K + scc[j];
+  }
+  float4v acc[8], accu[SWIGLU ? 8 : 1];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (SWIGLU) accu[j] = float4v{0.f, 0.f, 0.f, 0.f};
+  }
+  uint4 pre[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j]);
+  for (int k0 = 0; k0 < K; k0 += GG_KC) {
+    __syncthreads();                                     // the previous chunk is consumed
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(&rows[srr[j]][scc[j]]) = pre[j];
+    __syncthreads();
+    if (k0 + GG_KC < K) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j] + k0 + GG_KC);
+    }
+    if (wave_on) {
+#pragma unroll
+      for (int ks = 0; ks < GG_KC; ks += 32) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(wg + k0 + ks);
+        bf16x8 au;
+        if (SWIGLU) au = *reinterpret_cast<const bf16x8*>(wu + k0 + ks);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const bf16x8 b = *reinterpret_cast<const bf16x8*>(&rows[16 * j + fr][ks + fq * 8]);
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[j], 0, 0, 0);
+          if (SWIGLU) accu[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au, b, accu[j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!wave_on) return;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int r = r0 + 16 * j + fr;
+    if (r >= r1) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = nb + 4 * fq + i;
+      if (n < N) {
+        const float v = SWIGLU ? silu_f(acc[j][i]) * accu[j][i] : acc[j][i];
+        out[(size_t)r * N + n] = f2bf(v);
+      }
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const T* __restrict__ h, const T* __restrict__ y, const int* __restrict__ idx,
@@ -286,7 +380,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
     float* __restrict__ out) {
   const int t = blockIdx.x;
   const int* pos = plan + E + 2 + P;
-  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < d; c += gridDim.y * blockDim.x) {
     float s = 0.f;
     for (int k = 0; k < top; ++k) {
       const int p = t * top + k;
@@ -302,18 +396,19 @@ template <typename T>
 __global__ __launch_bounds__(256) void silu_mul_any_kernel(const T* __restrict__ x, int F,
                                                            T* __restrict__ y) {
   const size_t r = blockIdx.x;
-  for (int c = threadIdx.x; c < F; c += blockDim.x)
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < F; c += gridDim.y * blockDim.x)
     Act<T>::st(y + r * F + c,
                silu_f(Act<T>::ld(x + r * 2 * F + c)) * Act<T>::ld(x + r * 2 * F + F + c));
 }
 
 extern "C" int loqa_silu_mul_any(const void* x, int dt, int T, int F, void* y, hipStream_t st) {
   if (T <= 0) return 0;
+  const dim3 grid(T, T >= 512 ? 1 : (F + 255) / 256);
   if (dt == 0)
-    hipLaunchKernelGGL(silu_mul_any_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)x, F,
+    hipLaunchKernelGGL(silu_mul_any_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, F,
                        (bf16_t*)y);
   else
-    hipLaunchKernelGGL(silu_mul_any_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)x, F,
+    hipLaunchKernelGGL(silu_mul_any_kernel<float>, grid, dim3(256), 0, st, (const float*)x, F,
                        (float*)y);
   return (int)hipGetLastError();
 }
@@ -339,6 +434,17 @@ extern "C" int loqa_moe_grouped_gemm(const void* A, int dt, const void* W, const
                                      hipStream_t st) {
   if (P <= 0) return 0;
   const dim3 grid((P + GG_T - 1) / GG_T + E, (N + GG_T - 1) / GG_T);
+  if (dt == 0 && K % GG_KC == 0 && P >= 16 * (E > 0 ? E : 1) * 4 && P >= 1024) {
+    // prompt-sized: on average at least 64 rows per expert
+    const dim3 g2((P + GG_R2 - 1) / GG_R2 + E, (N + 63) / 64);
+    if (swiglu)
+      hipLaunchKernelGGL(moe_grouped_gemm_mfma2_kernel<1>, g2, dim3(256), 0, st, (const bf16_t*)A,
+                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
+    else
+      hipLaunchKernelGGL(moe_grouped_gemm_mfma2_kernel<0>, g2, dim3(256), 0, st, (const bf16_t*)A,
+                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
+    return (int)hipGetLastError();
+  }
   if (dt == 0 && K >= 32 && K % 32 == 0) {
     if (swiglu)
       hipLaunchKernelGGL(moe_grouped_gemm_mfma_kernel<1>, grid, dim3(256), 0, st, (const bf16_t*)A,
@@ -361,12 +467,13 @@ extern "C" int loqa_moe_combine(const void* h, const void* y, int dt, const void
                                 const void* wt, const void* plan, int T, int top, int E, int d,
                                 void* out, hipStream_t st) {
   if (T <= 0) return 0;
+  const dim3 cgrid(T, T >= 512 ? 1 : (d + 255) / 256);
   if (dt == 0)
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)h,
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, cgrid, dim3(256), 0, st, (const bf16_t*)h,
                        (const bf16_t*)y, (const int*)idx, (const float*)wt, (const int*)plan, T * top,
                        top, E, d, (float*)out);
   else
-    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)h,
+    hipLaunchKernelGGL(moe_combine_kernel<float>, cgrid, dim3(256), 0, st, (const float*)h,
                        (const float*)y, (const int*)idx, (const float*)wt, (const int*)plan, T * top,
                        top, E, d, (float*)out);
   return (int)hipGetLastError();

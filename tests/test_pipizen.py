@@ -412,14 +412,17 @@ def test_prompt_path_matches_folded_attention(full_model):
 
 
 @pytest.mark.gpu
-def test_grouped_expert_gemm_matrix_cores():
-    """The bf16 grouped expert GEMMs on the matrix cores (K a multiple of 32)
-    against the f32 reference: unequal expert loads, an empty expert, identity
-    experts, segments that do not fill a tile."""
+@pytest.mark.parametrize("T,d,F", [(333, 96, 64), (700, 128, 192), (2100, 64, 64)],
+                         ids=["direct", "staged", "staged_many_rows"])
+def test_grouped_expert_gemm_matrix_cores(T, d, F):
+    """The bf16 grouped expert GEMMs on the matrix cores (K a multiple of 32;
+    prompt-sized batches stage the token rows in LDS) against the f32
+    reference: unequal expert loads, an empty expert, identity experts,
+    segments that do not fill a tile."""
     from loqa_hub_amd.ops import reference as ref
     from loqa_hub_amd.ops import seqmix
     g = torch.Generator().manual_seed(3)
-    T, d, F, E, top = 333, 96, 64, 7, 3
+    E, top = 7, 3
     h = torch.randn(T, d, generator=g).to(torch.bfloat16)
     wgu = (torch.randn(E, 2 * F, d, generator=g) / d ** 0.5).to(torch.bfloat16)
     wd = (torch.randn(E, d, F, generator=g) / F ** 0.5).to(torch.bfloat16)
