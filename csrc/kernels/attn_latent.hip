@@ -198,6 +198,7 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_attn_kernel(LatAttnParams 
 // half of the wave takes half of the row, read two entries at a time, two
 // independent accumulators), and for P.C a lane owns pairs of output entries.
 #define LAT_MAXP 8      // R <= 128 * LAT_MAXP
+#define LAT_MAXCH 10    // 16-byte chunks of a key tile per thread
 
 template <typename T> struct Pair;
 template <> struct Pair<bf16_t> {
@@ -270,24 +271,74 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_attn2_kernel(LatAttnParams
   // the two halves of a row, in pairs: [0, hp) and [hp, W / 2)
   const int npair = W >> 1, hp = (npair + 1) >> 1;
   const int c_lo = half ? hp : 0, c_hi = half ? npair : hp;
+  // Staging. Rows that are multiples of 16 bytes move as 16-byte chunks: the
+  // tile's page lookups are done once (row offsets in LDS), then every thread
+  // issues its chunks back to back, and the NEXT tile's chunks are in flight in
+  // registers while this tile is scored. Other row sizes go 4 bytes at a time.
+  long long* rowoff = reinterpret_cast<long long*>(ktile + (size_t)KT * Ws);   // [KT]
+  const int epc = 16 / (int)sizeof(T);                  // entries per chunk
+  const bool vec = (W % epc) == 0;
+  const int cpr = W / epc, nch = KT * cpr;
+  uint4 pre[LAT_MAXCH];
+  auto plan_rows = [&](int kt) {
+    if (threadIdx.x < KT) {
+      const int key = kt + threadIdx.x;
+      rowoff[threadIdx.x] = key < k1
+          ? (long long)(((size_t)bt[key / p.blk] * p.blk + key % p.blk) * W) : -1ll;
+    }
+  };
+  auto fetch = [&]() {
+#pragma unroll
+    for (int j = 0; j < LAT_MAXCH; ++j) {
+      const int c = threadIdx.x + LAT_THREADS * j;
+      pre[j] = make_uint4(0, 0, 0, 0);
+      if (c < nch) {
+        const int row = c / cpr, cc = c - row * cpr;
+        const long long off = rowoff[row];
+        if (off >= 0) pre[j] = *reinterpret_cast<const uint4*>(cache + off + cc * epc);
+      }
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int j = 0; j < LAT_MAXCH; ++j) {
+      const int c = threadIdx.x + LAT_THREADS * j;
+      if (c < nch) {
+        const int row = c / cpr, cc = c - row * cpr;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(ktile + (size_t)row * Ws + cc * epc);
+        dst[0] = pre[j].x; dst[1] = pre[j].y; dst[2] = pre[j].z; dst[3] = pre[j].w;
+      }
+    }
+  };
+  if (vec && k0 < k1) {
+    plan_rows(k0);
+    __syncthreads();
+    fetch();
+  }
   for (int kt = k0; kt < k1; kt += KT) {
     __syncthreads();
-    for (int j = wave; j < KT; j += LAT_WAVES) {
-      const int key = kt + j;
-      uint32_t* dst = reinterpret_cast<uint32_t*>(ktile + (size_t)j * Ws);
-      if (key < k1) {
-        const T* src = cache + ((size_t)bt[key / p.blk] * p.blk + key % p.blk) * W;
-        if (sizeof(T) == 2) {
-          const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src);
-          for (int c = lane; c < npair; c += 64) dst[c] = s32[c];
-        } else {
-          const float* sf = reinterpret_cast<const float*>(src);
-          float* df = reinterpret_cast<float*>(dst);
-          for (int c = lane; c < W; c += 64) df[c] = sf[c];
+    if (vec) {
+      commit();
+      if (kt + KT < k1) plan_rows(kt + KT);
+    } else {
+      for (int j = wave; j < KT; j += LAT_WAVES) {
+        const int key = kt + j;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(ktile + (size_t)j * Ws);
+        if (key < k1) {
+          const T* src = cache + ((size_t)bt[key / p.blk] * p.blk + key % p.blk) * W;
+          if (sizeof(T) == 2) {
+            const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src);
+            for (int c = lane; c < npair; c += 64) dst[c] = s32[c];
+          } else {
+            const float* sf = reinterpret_cast<const float*>(src);
+            float* df = reinterpret_cast<float*>(dst);
+            for (int c = lane; c < W; c += 64) df[c] = sf[c];
+          }
         }
       }
     }
     __syncthreads();
+    if (vec && kt + KT < k1) fetch();
     float s = -INFINITY;
     const bool has = key_l < KT && kt + key_l < k1;
     if (has) {
@@ -425,10 +476,13 @@ extern "C" int loqa_latent_attention(
   if (W % 2 == 0 && R % 2 == 0 && R <= 128 * LAT_MAXP) {
     const size_t esz = dt == 0 ? 2 : 4;
     int KT2 = 32;
-    while (KT2 > 4 && (size_t)(LAT_WAVES * W + LAT_WAVES * KT2) * 4 + (size_t)KT2 * (W + 2) * esz > 60 * 1024)
+    const size_t chunks_per_row = ((size_t)W * esz + 15) / 16;
+    while (KT2 > 4 && ((size_t)(LAT_WAVES * W + LAT_WAVES * KT2) * 4 + (size_t)KT2 * (W + 2) * esz +
+                       KT2 * 8 > 60 * 1024 || KT2 * chunks_per_row > (size_t)LAT_THREADS * LAT_MAXCH))
       KT2 >>= 1;
-    const size_t smem2 = (size_t)(LAT_WAVES * W + LAT_WAVES * KT2) * 4 + (size_t)KT2 * (W + 2) * esz;
-    if (smem2 <= 64 * 1024) {
+    const size_t smem2 = (size_t)(LAT_WAVES * W + LAT_WAVES * KT2) * 4 + (size_t)KT2 * (W + 2) * esz +
+                         KT2 * 8 + 8;
+    if (smem2 <= 64 * 1024 && KT2 * chunks_per_row <= (size_t)LAT_THREADS * LAT_MAXCH) {
       p.KT = KT2;
       const dim3 grid2(T, (H + LAT_WAVES - 1) / LAT_WAVES, p.num_splits);
       if (dt == 0) hipLaunchKernelGGL(latent_attn2_kernel<bf16_t>, grid2, dim3(LAT_THREADS), smem2, st, p);

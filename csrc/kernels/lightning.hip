@@ -8,17 +8,20 @@
 // lightning_scan_kernel: one workgroup per (sequence, head, 32 value columns).
 // The columns of S evolve independently, so the grid splits Dv freely. A
 // thread holds S[d, e] for one column e and a contiguous run of MAXD rows d in
-// registers (8 threads per column). The step's tokens are staged TC at a time
-// in LDS (SiLU applied once, rows zero-padded to 8 MAXD so the recurrence reads
+// registers (16 threads per column, 8 waves: two per SIMD, so one wave's LDS and
+// cross-lane latencies hide behind the other's arithmetic). The step's tokens are staged TC at a time
+// in LDS (SiLU applied once, rows zero-padded to 16 MAXD so the recurrence reads
 // them as float4); the raw values of the next TC tokens are already in flight
 // in registers while the current ones are processed. The recurrence runs token
-// by token in f32 in the order of the definition; the 8 row-partials of o_t
-// are summed in a fixed order (pairs inside a wave, then the 4 waves). A prompt
+// by token in f32 in the order of the definition; the 16 row-partials of o_t
+// are summed in a fixed order (pairs inside a wave, then the 8 waves). A prompt
 // portion, a single decode token, or any cut of a prompt gives the same bits.
 #include "seqmix.h"
 
 #define LS_EC 32        // value columns per workgroup
-#define LS_DP 8         // row partitions (threads per column)
+#define LS_DP 16        // row partitions (threads per column)
+#define LS_THREADS (LS_EC * LS_DP)
+#define LS_WAVES (LS_THREADS / 64)
 
 template <typename T, int MAXD, int TC>   // D <= LS_DP * MAXD
 __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
@@ -26,13 +29,13 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
     const int* __restrict__ state_slots, const int* __restrict__ cu_q,
     const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ o) {
   constexpr int DPAD = LS_DP * MAXD;            // padded row length in LDS
-  constexpr int NPT = TC * DPAD / 256;          // staged q (and k) values per thread
-  constexpr int NVT = TC * LS_EC / 256;         // staged v values per thread
+  constexpr int NPT = TC * DPAD / LS_THREADS;   // staged q (and k) values per thread
+  constexpr int NVT = TC * LS_EC / LS_THREADS;  // staged v values per thread
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                         // [TC][DPAD]
   float* ks = qs + TC * DPAD;              // [TC][DPAD]
   float* vs = ks + TC * DPAD;              // [TC][EC]
-  float* red = vs + TC * LS_EC;            // [TC][4 waves][EC]
+  float* red = vs + TC * LS_EC;            // [TC][LS_WAVES][EC]
   const int b = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * LS_EC;
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
   if (q1 <= q0) return;
@@ -54,7 +57,7 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
   auto fetch = [&](int t0) {               // raw projections of tokens t0 .. t0 + TC
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
-      const int i = tid + 256 * j, tt = i / DPAD, d = i % DPAD;
+      const int i = tid + LS_THREADS * j, tt = i / DPAD, d = i % DPAD;
       const bool ok = t0 + tt < q1 && d < D;
       const T* row = qkv + (size_t)(ok ? t0 + tt : q0) * ld;
       rq[j] = ok ? Act<T>::ld(row + qoff + d) : 0.f;
@@ -62,7 +65,7 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
     }
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-      const int i = tid + 256 * j, tt = i / LS_EC, c = i % LS_EC;
+      const int i = tid + LS_THREADS * j, tt = i / LS_EC, c = i % LS_EC;
       const bool ok = t0 + tt < q1 && e0 + c < Dv;
       rv[j] = ok ? Act<T>::ld(qkv + (size_t)(t0 + tt) * ld + voff + c) : 0.f;
     }
@@ -73,11 +76,11 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
     __syncthreads();                       // the previous round's LDS is consumed
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
-      qs[tid + 256 * j] = silu_f(rq[j]);   // silu(0) = 0 keeps the padding zero
-      ks[tid + 256 * j] = silu_f(rk[j]);
+      qs[tid + LS_THREADS * j] = silu_f(rq[j]);   // silu(0) = 0 keeps the padding zero
+      ks[tid + LS_THREADS * j] = silu_f(rk[j]);
     }
 #pragma unroll
-    for (int j = 0; j < NVT; ++j) vs[tid + 256 * j] = silu_f(rv[j]);
+    for (int j = 0; j < NVT; ++j) vs[tid + LS_THREADS * j] = silu_f(rv[j]);
     __syncthreads();
     if (t0 + TC < q1) fetch(t0 + TC);      // in flight during the recurrence below
     // two tokens per trip: the second token's LDS reads and read-out sums are
@@ -99,15 +102,17 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
       }
       float part = (p0 + p1) + (p2 + p3);
       part += __shfl_xor(part, 32, 64);    // the wave's two row partitions
-      if (lane < 32) red[(tt * 4 + wave) * LS_EC + e] = part;
+      if (lane < 32) red[(tt * LS_WAVES + wave) * LS_EC + e] = part;
     }
     __syncthreads();
-    for (int i = tid; i < nt * LS_EC; i += 256) {
+    for (int i = tid; i < nt * LS_EC; i += LS_THREADS) {
       const int tt = i / LS_EC, c = i % LS_EC;
       if (e0 + c < Dv) {
-        const float* r = red + tt * 4 * LS_EC + c;
-        o[(size_t)(t0 + tt) * H * Dv + (size_t)h * Dv + e0 + c] =
-            ((r[0] + r[LS_EC]) + r[2 * LS_EC]) + r[3 * LS_EC];
+        const float* r = red + tt * LS_WAVES * LS_EC + c;
+        float sum = r[0];
+#pragma unroll
+        for (int w = 1; w < LS_WAVES; ++w) sum += r[w * LS_EC];
+        o[(size_t)(t0 + tt) * H * Dv + (size_t)h * Dv + e0 + c] = sum;
       }
     }
   }
@@ -141,17 +146,17 @@ extern "C" int loqa_lightning_scan(const void* qkv, int dt, long ld, int H, int 
                                    const void* cu_q, const void* positions, const void* decay,
                                    void* o, int B, int T, hipStream_t st) {
   if (T <= 0 || B <= 0) return 0;
-  if (D > LS_DP * 32 || D <= 0 || Dv <= 0) return (int)hipErrorInvalidValue;
+  if (D > LS_DP * 16 || D <= 0 || Dv <= 0) return (int)hipErrorInvalidValue;
   (void)nslots;
   const dim3 grid(B, H, (Dv + LS_EC - 1) / LS_EC), block(LS_EC * LS_DP);
 #define GO(TT, MD, TCC)                                                                          \
   hipLaunchKernelGGL((lightning_scan_kernel<TT, MD, TCC>), grid, block,                          \
-                     (size_t)(2 * TCC * LS_DP * MD + TCC * LS_EC + TCC * 4 * LS_EC) * 4, st,     \
+                     (size_t)(2 * TCC * LS_DP * MD + TCC * LS_EC + TCC * LS_WAVES * LS_EC) * 4, st, \
                      (const TT*)qkv, ld, H, D, Dv, (float*)state, (const int*)state_slots,       \
                      (const int*)cu_q, (const int*)positions, (const float*)decay, (float*)o)
-  const int md = D <= 64 ? 8 : (D <= 128 ? 16 : 32);
-  if (dt == 0) { if (md == 8) GO(bf16_t, 8, 32); else if (md == 16) GO(bf16_t, 16, 32); else GO(bf16_t, 32, 16); }
-  else { if (md == 8) GO(float, 8, 32); else if (md == 16) GO(float, 16, 32); else GO(float, 32, 16); }
+  const int md = D <= 64 ? 4 : (D <= 128 ? 8 : 16);
+  if (dt == 0) { if (md == 4) GO(bf16_t, 4, 16); else if (md == 8) GO(bf16_t, 8, 16); else GO(bf16_t, 16, 16); }
+  else { if (md == 4) GO(float, 4, 16); else if (md == 8) GO(float, 8, 16); else GO(float, 16, 16); }
 #undef GO
   return (int)hipGetLastError();
 }

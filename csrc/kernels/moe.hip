@@ -279,14 +279,17 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
   }
 }
 
-// Prompt-sized batches (hundreds of rows per expert): 128 token rows x 64
+// Prompt-sized batches (hundreds of rows per expert): 128 token rows x 128
 // features per workgroup, the token rows of a 64-wide K chunk staged once in
 // LDS for the 4 waves (the next chunk's rows already in flight in registers),
-// weights streamed straight from global memory - every weight fragment is
-// loaded once per workgroup and feeds 8 MFMAs, every staged row fragment 2
-// (gate and up). Same fragment layout and summation order as the kernel above.
+// weights streamed straight from global memory. A wave owns 2 feature
+// sub-tiles of 16 (and their up-rows for SwiGLU): every weight fragment is
+// loaded once per workgroup and feeds 8 MFMAs, every staged row fragment read
+// from LDS feeds 2 (4 with SwiGLU). Same fragment layout and summation order
+// as the kernel above.
 #define GG_R2 128
 #define GG_KC 64
+#define GG_NF 2
 
 template <int SWIGLU>
 __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
@@ -305,13 +308,18 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
   if (e == E) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int fr = lane & 15, fq = lane >> 4;
-  const int nb = blockIdx.y * 64 + wave * 16;
+  const int nb = blockIdx.y * (64 * GG_NF) + wave * (16 * GG_NF);
   const bool wave_on = nb < N;                           // idle waves still stage rows
   const int wrows = SWIGLU ? 2 * N : N;
   const bf16_t* We = Wt + (size_t)e * wrows * K;
-  const int nrow = min(nb + fr, N - 1);
-  const bf16_t* wg = We + (size_t)nrow * K + fq * 8;
-  const bf16_t* wu = SWIGLU ? We + (size_t)(N + nrow) * K + fq * 8 : nullptr;
+  const bf16_t* wg[GG_NF];
+  const bf16_t* wu[GG_NF];
+#pragma unroll
+  for (int f = 0; f < GG_NF; ++f) {
+    const int nrow = min(nb + 16 * f + fr, N - 1);
+    wg[f] = We + (size_t)nrow * K + fq * 8;
+    wu[f] = SWIGLU ? We + (size_t)(N + nrow) * K + fq * 8 : nullptr;
+  }
   // staging: thread -> 4 chunks of 8 entries: row = (tid + 256 j) / 8, column chunk = % 8
   const bf16_t* srow[4];
   int srr[4], scc[4];
@@ -324,12 +332,14 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
     const size_t src = SWIGLU ? (size_t)(perm[r] / top) : (size_t)r;
     srow[j] = A + src * K + scc[j];
   }
-  float4v acc[8], accu[SWIGLU ? 8 : 1];
+  float4v acc[GG_NF][8], accu[SWIGLU ? GG_NF : 1][SWIGLU ? 8 : 1];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
-    if (SWIGLU) accu[j] = float4v{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int f = 0; f < GG_NF; ++f)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      acc[f][j] = float4v{0.f, 0.f, 0.f, 0.f};
+      if (SWIGLU) accu[f][j] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
   uint4 pre[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j]);
@@ -345,32 +355,41 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
     if (wave_on) {
 #pragma unroll
       for (int ks = 0; ks < GG_KC; ks += 32) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(wg + k0 + ks);
-        bf16x8 au;
-        if (SWIGLU) au = *reinterpret_cast<const bf16x8*>(wu + k0 + ks);
+        bf16x8 a[GG_NF], au[GG_NF];
+#pragma unroll
+        for (int f = 0; f < GG_NF; ++f) {
+          a[f] = *reinterpret_cast<const bf16x8*>(wg[f] + k0 + ks);
+          if (SWIGLU) au[f] = *reinterpret_cast<const bf16x8*>(wu[f] + k0 + ks);
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const bf16x8 b = *reinterpret_cast<const bf16x8*>(&rows[16 * j + fr][ks + fq * 8]);
-          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[j], 0, 0, 0);
-          if (SWIGLU) accu[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au, b, accu[j], 0, 0, 0);
+#pragma unroll
+          for (int f = 0; f < GG_NF; ++f) {
+            acc[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[f], b, acc[f][j], 0, 0, 0);
+            if (SWIGLU)
+              accu[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au[f], b, accu[f][j], 0, 0, 0);
+          }
         }
       }
     }
   }
   if (!wave_on) return;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int r = r0 + 16 * j + fr;
-    if (r >= r1) continue;
+  for (int f = 0; f < GG_NF; ++f)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = nb + 4 * fq + i;
-      if (n < N) {
-        const float v = SWIGLU ? silu_f(acc[j][i]) * accu[j][i] : acc[j][i];
-        out[(size_t)r * N + n] = f2bf(v);
+    for (int j = 0; j < 8; ++j) {
+      const int r = r0 + 16 * j + fr;
+      if (r >= r1) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = nb + 16 * f + 4 * fq + i;
+        if (n < N) {
+          const float v = SWIGLU ? silu_f(acc[f][j][i]) * accu[f][j][i] : acc[f][j][i];
+          out[(size_t)r * N + n] = f2bf(v);
+        }
       }
     }
-  }
 }
 
 template <typename T>
@@ -436,7 +455,7 @@ extern "C" int loqa_moe_grouped_gemm(const void* A, int dt, const void* W, const
   const dim3 grid((P + GG_T - 1) / GG_T + E, (N + GG_T - 1) / GG_T);
   if (dt == 0 && K % GG_KC == 0 && P >= 16 * (E > 0 ? E : 1) * 4 && P >= 1024) {
     // prompt-sized: on average at least 64 rows per expert
-    const dim3 g2((P + GG_R2 - 1) / GG_R2 + E, (N + 63) / 64);
+    const dim3 g2((P + GG_R2 - 1) / GG_R2 + E, (N + 64 * GG_NF - 1) / (64 * GG_NF));
     if (swiglu)
       hipLaunchKernelGGL(moe_grouped_gemm_mfma2_kernel<1>, g2, dim3(256), 0, st, (const bf16_t*)A,
                          (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
