@@ -345,7 +345,8 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_attn2_kernel(LatAttnParams
       const T* kr = ktile + (size_t)key_l * Ws;
       const float* q = qs + wave * W;
       float a0 = 0.f, a1 = 0.f;
-      for (int c = c_lo; c < c_hi; ++c) {
+#pragma unroll 8
+      for (int c = c_lo; c < c_hi; ++c) {    // 8 pairs in flight: LDS latency overlaps the FMAs
         const float2 kk = Pair<T>::ld(kr + 2 * c);
         const float2 qq = *reinterpret_cast<const float2*>(q + 2 * c);
         a0 += qq.x * kk.x;
@@ -367,6 +368,7 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_attn2_kernel(LatAttnParams
 #pragma unroll
     for (int i = 0; i < LAT_MAXP; ++i) { acc[i].x *= corr; acc[i].y *= corr; }
     const int nj = min(KT, k1 - kt);
+#pragma unroll 4
     for (int j = 0; j < nj; ++j) {
       const float pv = ps[wave * KT + j];
       const T* cr = ktile + (size_t)j * Ws;

@@ -12,7 +12,7 @@ __global__ __launch_bounds__(256) void dyt_norm_kernel(
   const int r = blockIdx.x;
   const size_t src = (size_t)(row_idx ? row_idx[r] : r) * d;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < d; c += gridDim.y * blockDim.x)
-    Act<TO>::st(y + (size_t)r * d + c, tanhf(alpha * Act<TI>::ld(x + src + c)) * w[c] + b[c]);
+    Act<TO>::st(y + (size_t)r * d + c, tanh_f(alpha * Act<TI>::ld(x + src + c)) * w[c] + b[c]);
 }
 
 template <typename TY, typename TO>
@@ -22,9 +22,9 @@ __global__ __launch_bounds__(256) void dyt_add_norm_kernel(
     const float* __restrict__ b2, float a2, TO* __restrict__ h, int d) {
   const size_t base = (size_t)blockIdx.x * d;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < d; c += gridDim.y * blockDim.x) {
-    const float v = resid[base + c] + (tanhf(a1 * Act<TY>::ld(y + base + c)) * w1[c] + b1[c]);
+    const float v = resid[base + c] + (tanh_f(a1 * Act<TY>::ld(y + base + c)) * w1[c] + b1[c]);
     resid[base + c] = v;
-    if (h) Act<TO>::st(h + base + c, tanhf(a2 * v) * w2[c] + b2[c]);
+    if (h) Act<TO>::st(h + base + c, tanh_f(a2 * v) * w2[c] + b2[c]);
   }
 }
 
