@@ -77,21 +77,39 @@ __global__ __launch_bounds__(LP_THREADS) void latent_prefill_kernel(LatPrefillPa
   const bf16_t* kbase = p.k + (size_t)k0 * kst + (size_t)head * DK;
   const bf16_t* vbase = p.v + (size_t)k0 * vst + (size_t)head * DV;
 
+  // K / V tiles go through registers: the next tile's 16-byte chunks are
+  // requested before this tile's math and stored to LDS after it
+  constexpr int NKC = LP_TILE * CHK / LP_THREADS, NVC = LP_TILE * CHV / LP_THREADS;
+  uint4 pk[NKC], pv[NVC];
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < NKC; ++j) {
+      const int c = threadIdx.x + LP_THREADS * j, kr = c / CHK, cc = (c - kr * CHK) * 8;
+      pk[j] = kt + kr < kend ? *reinterpret_cast<const uint4*>(kbase + (size_t)(kt + kr) * kst + cc)
+                             : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < NVC; ++j) {
+      const int c = threadIdx.x + LP_THREADS * j, kr = c / CHV, cc = (c - kr * CHV) * 8;
+      pv[j] = kt + kr < kend ? *reinterpret_cast<const uint4*>(vbase + (size_t)(kt + kr) * vst + cc)
+                             : make_uint4(0, 0, 0, 0);
+    }
+  };
+  fetch(0);
   for (int kt = 0; kt < kend; kt += LP_TILE) {
     __syncthreads();
-    for (int c = threadIdx.x; c < LP_TILE * CHK; c += LP_THREADS) {
-      const int kr = c / CHK, cc = (c - kr * CHK) * 8;
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (kt + kr < kend) x = *reinterpret_cast<const uint4*>(kbase + (size_t)(kt + kr) * kst + cc);
-      *reinterpret_cast<uint4*>(&sm.k[kr][cc]) = x;
+#pragma unroll
+    for (int j = 0; j < NKC; ++j) {
+      const int c = threadIdx.x + LP_THREADS * j, kr = c / CHK, cc = (c - kr * CHK) * 8;
+      *reinterpret_cast<uint4*>(&sm.k[kr][cc]) = pk[j];
     }
-    for (int c = threadIdx.x; c < LP_TILE * CHV; c += LP_THREADS) {
-      const int kr = c / CHV, cc = (c - kr * CHV) * 8;
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (kt + kr < kend) x = *reinterpret_cast<const uint4*>(vbase + (size_t)(kt + kr) * vst + cc);
-      *reinterpret_cast<uint4*>(&sm.v[kr][cc]) = x;
+#pragma unroll
+    for (int j = 0; j < NVC; ++j) {
+      const int c = threadIdx.x + LP_THREADS * j, kr = c / CHV, cc = (c - kr * CHV) * 8;
+      *reinterpret_cast<uint4*>(&sm.v[kr][cc]) = pv[j];
     }
     __syncthreads();
+    if (kt + LP_TILE < kend) fetch(kt + LP_TILE);
 
     float16v st[2];
 #pragma unroll

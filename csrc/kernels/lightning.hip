@@ -5,42 +5,55 @@
 // q, k, v = SiLU of the projection columns. S [D, Dv] lives in f32 state slots
 // between steps.
 //
-// lightning_scan_kernel: one workgroup per (sequence, head, 32 value columns).
-// The columns of S evolve independently, so the grid splits Dv freely. A
+// lightning_prep_kernel: act = SiLU of the q | k | v projection columns, f32,
+// once per step (every column block of a head reads the same q and k).
+//
+// lightning_scan_kernel: one workgroup per (sequence, head, EC value columns).
+// The columns of S evolve independently, so the grid splits Dv freely: EC is
+// 32 when the batch alone fills the GPU and 16 or 8 for a lone prompt. A
 // thread holds S[d, e] for one column e and a contiguous run of MAXD rows d in
-// registers (16 threads per column, 8 waves: two per SIMD, so one wave's LDS and
-// cross-lane latencies hide behind the other's arithmetic). The step's tokens are staged TC at a time
-// in LDS (SiLU applied once, rows zero-padded to 16 MAXD so the recurrence reads
-// them as float4); the raw values of the next TC tokens are already in flight
-// in registers while the current ones are processed. The recurrence runs token
-// by token in f32 in the order of the definition; the 16 row-partials of o_t
-// are summed in a fixed order (pairs inside a wave, then the 8 waves). A prompt
-// portion, a single decode token, or any cut of a prompt gives the same bits.
+// registers (16 threads per column). The step's tokens are staged TC at a time
+// in LDS (rows zero-padded to 16 MAXD so the recurrence reads them as float4);
+// the values of the next two rounds are already in flight in registers while
+// the current one is processed. The recurrence runs token by token in f32 in
+// the order of the definition; only the S updates chain from token to token,
+// the next token's k / q / v are read from LDS while this token is computed,
+// and the 16 row-partials of o_t are written to LDS and summed in a fixed
+// order after each round. A prompt portion, a single decode token, or any cut
+// of a prompt gives the same bits (for a given EC: the column split does not
+// change any sum).
 #include "seqmix.h"
+#include <type_traits>
 
-#define LS_EC 32        // value columns per workgroup
 #define LS_DP 16        // row partitions (threads per column)
-#define LS_THREADS (LS_EC * LS_DP)
-#define LS_WAVES (LS_THREADS / 64)
 
-template <typename T, int MAXD, int TC>   // D <= LS_DP * MAXD
-__global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
-    const T* __restrict__ qkv, long ld, int H, int D, int Dv, float* __restrict__ state,
+template <typename T>
+__global__ __launch_bounds__(256) void lightning_prep_kernel(const T* __restrict__ qkv, long ld,
+                                                             int n, float* __restrict__ act) {
+  const size_t r = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < n; c += gridDim.y * blockDim.x)
+    act[r * n + c] = silu_f(Act<T>::ld(qkv + r * ld + c));
+}
+
+template <int MAXD, int TC, int EC>   // D <= LS_DP * MAXD
+__global__ __launch_bounds__(EC * LS_DP) void lightning_scan_kernel(
+    const float* __restrict__ act, long ld, int H, int D, int Dv, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q,
     const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ o) {
+  constexpr int NTH = EC * LS_DP;
   constexpr int DPAD = LS_DP * MAXD;            // padded row length in LDS
-  constexpr int NPT = TC * DPAD / LS_THREADS;   // staged q (and k) values per thread
-  constexpr int NVT = TC * LS_EC / LS_THREADS;  // staged v values per thread
+  constexpr int NPT = TC * DPAD / NTH;          // staged q (and k) values per thread
+  constexpr int NVT = (TC * EC + NTH - 1) / NTH;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                         // [TC][DPAD]
   float* ks = qs + TC * DPAD;              // [TC][DPAD]
   float* vs = ks + TC * DPAD;              // [TC][EC]
-  float* red = vs + TC * LS_EC;            // [TC][LS_WAVES][EC]
-  const int b = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * LS_EC;
+  float* red = vs + TC * EC;               // [TC][LS_DP][EC]
+  const int b = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * EC;
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
   if (q1 <= q0) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int e = tid % LS_EC, dp = tid / LS_EC;
+  const int tid = threadIdx.x;
+  const int e = tid % EC, dp = tid / EC;
   const bool col = e0 + e < Dv;
   const float lam = decay[h];
   float* Sg = state + (((size_t)state_slots[b] * H + h) * D) * Dv + e0 + e;
@@ -53,68 +66,92 @@ __global__ __launch_bounds__(LS_EC * LS_DP) void lightning_scan_kernel(
   }
   const size_t qoff = (size_t)h * D, koff = (size_t)H * D + (size_t)h * D;
   const size_t voff = 2 * (size_t)H * D + (size_t)h * Dv + e0;
-  float rq[NPT], rk[NPT], rv[NVT];
-  auto fetch = [&](int t0) {               // raw projections of tokens t0 .. t0 + TC
+  // Two register sets: while round r is processed, the loads of rounds r + 1
+  // and r + 2 are in flight.
+  float rq[2][NPT], rk[2][NPT], rv[2][NVT];
+  auto fetch = [&](auto BUF, int t0) {     // activations of tokens t0 .. t0 + TC
+    constexpr int U = decltype(BUF)::value;
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
-      const int i = tid + LS_THREADS * j, tt = i / DPAD, d = i % DPAD;
+      const int i = tid + NTH * j, tt = i / DPAD, d = i % DPAD;
       const bool ok = t0 + tt < q1 && d < D;
-      const T* row = qkv + (size_t)(ok ? t0 + tt : q0) * ld;
-      rq[j] = ok ? Act<T>::ld(row + qoff + d) : 0.f;
-      rk[j] = ok ? Act<T>::ld(row + koff + d) : 0.f;
+      const float* row = act + (size_t)(ok ? t0 + tt : q0) * ld;
+      rq[U][j] = ok ? row[qoff + d] : 0.f;
+      rk[U][j] = ok ? row[koff + d] : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-      const int i = tid + LS_THREADS * j, tt = i / LS_EC, c = i % LS_EC;
-      const bool ok = t0 + tt < q1 && e0 + c < Dv;
-      rv[j] = ok ? Act<T>::ld(qkv + (size_t)(t0 + tt) * ld + voff + c) : 0.f;
+      const int i = tid + NTH * j, tt = i / EC, c = i % EC;
+      const bool ok = i < TC * EC && t0 + tt < q1 && e0 + c < Dv;
+      rv[U][j] = ok ? act[(size_t)(t0 + tt) * ld + voff + c] : 0.f;
     }
   };
-  fetch(q0);
-  for (int t0 = q0; t0 < q1; t0 += TC) {
+  auto round = [&](auto BUF, int t0) {
+    constexpr int U = decltype(BUF)::value;
     const int nt = min(TC, q1 - t0);
     __syncthreads();                       // the previous round's LDS is consumed
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
-      qs[tid + LS_THREADS * j] = silu_f(rq[j]);   // silu(0) = 0 keeps the padding zero
-      ks[tid + LS_THREADS * j] = silu_f(rk[j]);
+      qs[tid + NTH * j] = rq[U][j];
+      ks[tid + NTH * j] = rk[U][j];
     }
 #pragma unroll
-    for (int j = 0; j < NVT; ++j) vs[tid + LS_THREADS * j] = silu_f(rv[j]);
+    for (int j = 0; j < NVT; ++j)
+      if (tid + NTH * j < TC * EC) vs[tid + NTH * j] = rv[U][j];
     __syncthreads();
-    if (t0 + TC < q1) fetch(t0 + TC);      // in flight during the recurrence below
-    // two tokens per trip: the second token's LDS reads and read-out sums are
-    // independent of the first's, so they overlap its latency (only the S
-    // updates chain); four partial sums per token in a fixed order
-#pragma unroll 2
+    if (t0 + 2 * TC < q1) fetch(BUF, t0 + 2 * TC);   // this set is free again
+    float4 kc[MAXD / 4], qc[MAXD / 4];
+    float vc;
+    {
+      const float4* k4 = reinterpret_cast<const float4*>(ks + dp * MAXD);
+      const float4* q4 = reinterpret_cast<const float4*>(qs + dp * MAXD);
+#pragma unroll
+      for (int i = 0; i < MAXD / 4; ++i) { kc[i] = k4[i]; qc[i] = q4[i]; }
+      vc = vs[e];
+    }
     for (int tt = 0; tt < nt; ++tt) {
-      const float v = vs[tt * LS_EC + e];
-      const float4* k4 = reinterpret_cast<const float4*>(ks + tt * DPAD + dp * MAXD);
-      const float4* q4 = reinterpret_cast<const float4*>(qs + tt * DPAD + dp * MAXD);
+      float4 kn[MAXD / 4], qn[MAXD / 4];
+      float vn = 0.f;
+      const int tn = tt + 1 < nt ? tt + 1 : tt;          // clamped: the last read is a repeat
+      {
+        const float4* k4 = reinterpret_cast<const float4*>(ks + tn * DPAD + dp * MAXD);
+        const float4* q4 = reinterpret_cast<const float4*>(qs + tn * DPAD + dp * MAXD);
+#pragma unroll
+        for (int i = 0; i < MAXD / 4; ++i) { kn[i] = k4[i]; qn[i] = q4[i]; }
+        vn = vs[tn * EC + e];
+      }
       float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
       for (int i = 0; i < MAXD / 4; ++i) {
-        const float4 kk = k4[i], qq = q4[i];
-        S[4 * i] = lam * S[4 * i] + kk.x * v;         p0 += S[4 * i] * qq.x;
-        S[4 * i + 1] = lam * S[4 * i + 1] + kk.y * v; p1 += S[4 * i + 1] * qq.y;
-        S[4 * i + 2] = lam * S[4 * i + 2] + kk.z * v; p2 += S[4 * i + 2] * qq.z;
-        S[4 * i + 3] = lam * S[4 * i + 3] + kk.w * v; p3 += S[4 * i + 3] * qq.w;
+        S[4 * i] = lam * S[4 * i] + kc[i].x * vc;         p0 += S[4 * i] * qc[i].x;
+        S[4 * i + 1] = lam * S[4 * i + 1] + kc[i].y * vc; p1 += S[4 * i + 1] * qc[i].y;
+        S[4 * i + 2] = lam * S[4 * i + 2] + kc[i].z * vc; p2 += S[4 * i + 2] * qc[i].z;
+        S[4 * i + 3] = lam * S[4 * i + 3] + kc[i].w * vc; p3 += S[4 * i + 3] * qc[i].w;
       }
-      float part = (p0 + p1) + (p2 + p3);
-      part += __shfl_xor(part, 32, 64);    // the wave's two row partitions
-      if (lane < 32) red[(tt * LS_WAVES + wave) * LS_EC + e] = part;
+      red[(tt * LS_DP + dp) * EC + e] = (p0 + p1) + (p2 + p3);
+#pragma unroll
+      for (int i = 0; i < MAXD / 4; ++i) { kc[i] = kn[i]; qc[i] = qn[i]; }
+      vc = vn;
     }
     __syncthreads();
-    for (int i = tid; i < nt * LS_EC; i += LS_THREADS) {
-      const int tt = i / LS_EC, c = i % LS_EC;
+    for (int i = tid; i < nt * EC; i += NTH) {
+      const int tt = i / EC, c = i % EC;
       if (e0 + c < Dv) {
-        const float* r = red + tt * LS_WAVES * LS_EC + c;
+        const float* r = red + tt * LS_DP * EC + c;
         float sum = r[0];
 #pragma unroll
-        for (int w = 1; w < LS_WAVES; ++w) sum += r[w * LS_EC];
+        for (int w = 1; w < LS_DP; ++w) sum += r[w * EC];
         o[(size_t)(t0 + tt) * H * Dv + (size_t)h * Dv + e0 + c] = sum;
       }
     }
+  };
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  fetch(B0{}, q0);
+  if (q0 + TC < q1) fetch(B1{}, q0 + TC);
+  for (int t0 = q0; t0 < q1; t0 += 2 * TC) {
+    round(B0{}, t0);
+    if (t0 + TC < q1) round(B1{}, t0 + TC);
   }
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) {
@@ -141,22 +178,45 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(
     Act<TO>::st(y + r * n + c, o[r * n + c] * inv * w[c] * sigmoid_f(Act<TG>::ld(gate + r * ldg + c)));
 }
 
-extern "C" int loqa_lightning_scan(const void* qkv, int dt, long ld, int H, int D, int Dv,
-                                   void* state, int nslots, const void* state_slots,
-                                   const void* cu_q, const void* positions, const void* decay,
-                                   void* o, int B, int T, hipStream_t st) {
+extern "C" int loqa_lightning_prep(const void* qkv, int dt, long ld, int T, int n, void* act,
+                                   hipStream_t st) {
+  if (T <= 0 || n <= 0) return 0;
+  const dim3 grid(T, T >= 512 ? 1 : (n + 255) / 256);
+  if (dt == 0)
+    hipLaunchKernelGGL(lightning_prep_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)qkv, ld, n,
+                       (float*)act);
+  else
+    hipLaunchKernelGGL(lightning_prep_kernel<float>, grid, dim3(256), 0, st, (const float*)qkv, ld, n,
+                       (float*)act);
+  return (int)hipGetLastError();
+}
+
+// act: f32 [T, >= 2 H D + H Dv] = SiLU'd q | k | v (lightning_prep).
+extern "C" int loqa_lightning_scan(const void* act, long ld, int H, int D, int Dv, void* state,
+                                   int nslots, const void* state_slots, const void* cu_q,
+                                   const void* positions, const void* decay, void* o, int B, int T,
+                                   hipStream_t st) {
   if (T <= 0 || B <= 0) return 0;
   if (D > LS_DP * 16 || D <= 0 || Dv <= 0) return (int)hipErrorInvalidValue;
   (void)nslots;
-  const dim3 grid(B, H, (Dv + LS_EC - 1) / LS_EC), block(LS_EC * LS_DP);
-#define GO(TT, MD, TCC)                                                                          \
-  hipLaunchKernelGGL((lightning_scan_kernel<TT, MD, TCC>), grid, block,                          \
-                     (size_t)(2 * TCC * LS_DP * MD + TCC * LS_EC + TCC * LS_WAVES * LS_EC) * 4, st, \
-                     (const TT*)qkv, ld, H, D, Dv, (float*)state, (const int*)state_slots,       \
+  // column block: 32 when (sequences x heads x column blocks) fill the GPU,
+  // narrower for a lone prompt
+  const long wg32 = (long)B * H * ((Dv + 31) / 32);
+  const int ec = wg32 >= 192 ? 32 : (wg32 * 2 >= 192 ? 16 : 8);
+#define GO(MD, TCC, ECC)                                                                          \
+  hipLaunchKernelGGL((lightning_scan_kernel<MD, TCC, ECC>), dim3(B, H, (Dv + ECC - 1) / ECC),     \
+                     dim3(ECC * LS_DP),                                                           \
+                     (size_t)(2 * TCC * LS_DP * MD + TCC * ECC + TCC * LS_DP * ECC) * 4, st,      \
+                     (const float*)act, ld, H, D, Dv, (float*)state, (const int*)state_slots,     \
                      (const int*)cu_q, (const int*)positions, (const float*)decay, (float*)o)
-  const int md = D <= 64 ? 4 : (D <= 128 ? 8 : 16);
-  if (dt == 0) { if (md == 4) GO(bf16_t, 4, 16); else if (md == 8) GO(bf16_t, 8, 16); else GO(bf16_t, 16, 16); }
-  else { if (md == 4) GO(float, 4, 16); else if (md == 8) GO(float, 8, 16); else GO(float, 16, 16); }
+#define GOE(MD, TCC)                                                                              \
+  do {                                                                                            \
+    if (ec == 32) GO(MD, TCC, 32); else if (ec == 16) GO(MD, TCC, 16); else GO(MD, TCC, 8);       \
+  } while (0)
+  if (D <= 64) GOE(4, 16);
+  else if (D <= 128) GOE(8, 16);
+  else GOE(16, 8);
+#undef GOE
 #undef GO
   return (int)hipGetLastError();
 }

@@ -343,35 +343,57 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
   uint4 pre[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j]);
+  // this chunk's weight fragments (2 k-steps); the next chunk's are requested
+  // before this chunk's MFMAs, so the weight stream's latency stays hidden
+  bf16x8 wa[2][GG_NF], wb[SWIGLU ? 2 : 1][GG_NF];
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int f = 0; f < GG_NF; ++f) {
+      wa[q][f] = *reinterpret_cast<const bf16x8*>(wg[f] + 32 * q);
+      if (SWIGLU) wb[q][f] = *reinterpret_cast<const bf16x8*>(wu[f] + 32 * q);
+    }
   for (int k0 = 0; k0 < K; k0 += GG_KC) {
     __syncthreads();                                     // the previous chunk is consumed
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(&rows[srr[j]][scc[j]]) = pre[j];
     __syncthreads();
-    if (k0 + GG_KC < K) {
+    const bool more = k0 + GG_KC < K;
+    bf16x8 na[2][GG_NF], nb2[SWIGLU ? 2 : 1][GG_NF];
+    if (more) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j] + k0 + GG_KC);
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int f = 0; f < GG_NF; ++f) {
+          na[q][f] = *reinterpret_cast<const bf16x8*>(wg[f] + k0 + GG_KC + 32 * q);
+          if (SWIGLU) nb2[q][f] = *reinterpret_cast<const bf16x8*>(wu[f] + k0 + GG_KC + 32 * q);
+        }
     }
     if (wave_on) {
 #pragma unroll
-      for (int ks = 0; ks < GG_KC; ks += 32) {
-        bf16x8 a[GG_NF], au[GG_NF];
-#pragma unroll
-        for (int f = 0; f < GG_NF; ++f) {
-          a[f] = *reinterpret_cast<const bf16x8*>(wg[f] + k0 + ks);
-          if (SWIGLU) au[f] = *reinterpret_cast<const bf16x8*>(wu[f] + k0 + ks);
-        }
+      for (int q = 0; q < 2; ++q) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const bf16x8 b = *reinterpret_cast<const bf16x8*>(&rows[16 * j + fr][ks + fq * 8]);
+          const bf16x8 b = *reinterpret_cast<const bf16x8*>(&rows[16 * j + fr][32 * q + fq * 8]);
 #pragma unroll
           for (int f = 0; f < GG_NF; ++f) {
-            acc[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[f], b, acc[f][j], 0, 0, 0);
+            acc[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[q][f], b, acc[f][j], 0, 0, 0);
             if (SWIGLU)
-              accu[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au[f], b, accu[f][j], 0, 0, 0);
+              accu[f][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[q][f], b, accu[f][j], 0, 0, 0);
           }
         }
       }
+    }
+    if (more) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int f = 0; f < GG_NF; ++f) {
+          wa[q][f] = na[q][f];
+          if (SWIGLU) wb[q][f] = nb2[q][f];
+        }
     }
   }
   if (!wave_on) return;

@@ -971,7 +971,7 @@ class LLMEngine:
         leading live sequences + flash prefill for the prompt chunks (adds
         ``cu_tail`` to ``host``), else None."""
         nd = sum(1 for k in kinds if k == 0)
-        if self.hybrid:
+        if getattr(self, "hybrid", False):
             return None      # one attention launch serves decode rows and chunks
         if (not self.MIXED_SPLIT or nd == 0 or nd == len(kinds)
                 or any(k != 0 for k in kinds[:nd])):

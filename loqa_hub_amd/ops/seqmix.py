@@ -141,7 +141,7 @@ def latent_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Tensor, cu
     assert cu_q.numel() == B + 1 and block_tables.shape[0] == B and positions.numel() >= T
     # few query rows over a long context: split the keys over workgroups
     hg = (H + 3) // 4
-    ns = 1 if T * hg >= 512 else max(1, min(32, -(-int(max_ctx) // 256), 1024 // max(1, T * hg)))
+    ns = 1 if T * hg >= 512 else max(1, min(32, -(-int(max_ctx) // 128), 1024 // max(1, T * hg)))
     ws = torch.empty(ns * T * H * (R + 2), dtype=torch.float32, device=qa.device) if ns > 1 else None
     if T:
         check(kernels().loqa_latent_attention(
@@ -250,10 +250,15 @@ def lightning_scan(qkv: torch.Tensor, H: int, D: int, Dv: int, state: torch.Tens
     assert cu_q.numel() == B + 1
     o = torch.empty(T, H * Dv, dtype=torch.float32, device=qkv.device)
     if T:
-        check(kernels().loqa_lightning_scan(
-            ptr(qkv), _dt(qkv), qkv.stride(0), H, D, Dv, ptr(state), state.shape[0],
-            ptr(state_slots), ptr(cu_q), ptr(positions), ptr(decay), ptr(o), B, T,
-            stream_ptr(qkv)), "lightning_scan")
+        # SiLU of q | k | v once, in f32 (every column block of a head shares q and k)
+        n = 2 * H * D + H * Dv
+        act = torch.empty(T, n, dtype=torch.float32, device=qkv.device)
+        k, st = kernels(), stream_ptr(qkv)
+        check(k.loqa_lightning_prep(ptr(qkv), _dt(qkv), qkv.stride(0), T, n, ptr(act), st),
+              "lightning_prep")
+        check(k.loqa_lightning_scan(ptr(act), n, H, D, Dv, ptr(state), state.shape[0],
+                                    ptr(state_slots), ptr(cu_q), ptr(positions), ptr(decay), ptr(o),
+                                    B, T, st), "lightning_scan")
     return o
 
 
