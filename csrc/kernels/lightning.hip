@@ -14,12 +14,12 @@
 // thread holds S[d, e] for one column e and a contiguous run of MAXD rows d in
 // registers (16 threads per column). The step's tokens are staged TC at a time
 // in LDS (rows zero-padded to 16 MAXD so the recurrence reads them as float4);
-// the values of the next two rounds are already in flight in registers while
+// the values of the next two token groups are already in flight in registers while
 // the current one is processed. The recurrence runs token by token in f32 in
 // the order of the definition; only the S updates chain from token to token,
 // the next token's k / q / v are read from LDS while this token is computed,
 // and the 16 row-partials of o_t are written to LDS and summed in a fixed
-// order after each round. A prompt portion, a single decode token, or any cut
+// order after each group. A prompt portion, a single decode token, or any cut
 // of a prompt gives the same bits (for a given EC: the column split does not
 // change any sum).
 #include "seqmix.h"
@@ -66,8 +66,8 @@ __global__ __launch_bounds__(EC * LS_DP) void lightning_scan_kernel(
   }
   const size_t qoff = (size_t)h * D, koff = (size_t)H * D + (size_t)h * D;
   const size_t voff = 2 * (size_t)H * D + (size_t)h * Dv + e0;
-  // Two register sets: while round r is processed, the loads of rounds r + 1
-  // and r + 2 are in flight.
+  // Two register sets: while token group g is processed, the loads of groups
+  // g + 1 and g + 2 are in flight.
   float rq[2][NPT], rk[2][NPT], rv[2][NVT];
   auto fetch = [&](auto BUF, int t0) {     // activations of tokens t0 .. t0 + TC
     constexpr int U = decltype(BUF)::value;
@@ -86,10 +86,10 @@ __global__ __launch_bounds__(EC * LS_DP) void lightning_scan_kernel(
       rv[U][j] = ok ? act[(size_t)(t0 + tt) * ld + voff + c] : 0.f;
     }
   };
-  auto round = [&](auto BUF, int t0) {
+  auto group = [&](auto BUF, int t0) {
     constexpr int U = decltype(BUF)::value;
     const int nt = min(TC, q1 - t0);
-    __syncthreads();                       // the previous round's LDS is consumed
+    __syncthreads();                       // the previous group's LDS is consumed
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
       qs[tid + NTH * j] = rq[U][j];
@@ -150,8 +150,8 @@ __global__ __launch_bounds__(EC * LS_DP) void lightning_scan_kernel(
   fetch(B0{}, q0);
   if (q0 + TC < q1) fetch(B1{}, q0 + TC);
   for (int t0 = q0; t0 < q1; t0 += 2 * TC) {
-    round(B0{}, t0);
-    if (t0 + TC < q1) round(B1{}, t0 + TC);
+    group(B0{}, t0);
+    if (t0 + TC < q1) group(B1{}, t0 + TC);
   }
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) {
