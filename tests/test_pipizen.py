@@ -93,6 +93,8 @@ def test_registry_reads_config(full_model):
     (O.latent(), None),                                                   # sink, YaRN, folded q/k
     (O.latent(heads=1, dim=32, rot_dim=4, vdim=8, kv_rank=16, dims=2), None),   # rot.dims < rot_dim
     (O.latent(scaling=False, base=500.0), None),
+    (O.latent(heads=2, dim=8, rot_dim=6, vdim=10, kv_rank=23, dims=4), None),    # odd row length
+    (O.latent(heads=5, dim=8, rot_dim=8, vdim=6, kv_rank=26), None),   # rows not 16-byte multiples
     (O.lightning_layer(), None),
     (O.lightning_layer(heads=1, dim=72, vdim=80, decay=[0.999]), None),   # D, Dv beyond one tile
     (O.lightning_layer(heads=5, dim=8, vdim=8, decay=[0.1, 0.3, 0.6, 0.9, 1.0]), None),
@@ -100,7 +102,7 @@ def test_registry_reads_config(full_model):
     (O.lightning_layer(), O.moe_ff()),
     (O.lightning_layer(), O.moe_ff(experts=4, identity=4, top=3, count=2, keep=1, shared=0)),
     (O.lightning_layer(), O.moe_ff(experts=70, identity=2, top=4, count=8, keep=3, ff=8)),
-], ids=["latent", "latent_partrot", "latent_plain", "lightning", "lightning_wide",
+], ids=["latent", "latent_partrot", "latent_plain", "latent_odd", "latent_unaligned", "lightning", "lightning_wide",
         "lightning_decays", "dense", "moe", "moe_identity", "moe_many"])
 def test_single_layer(device, layer):
     cfg = O.make_config([layer], width=40, vocab=90)
@@ -433,3 +435,35 @@ def test_grouped_expert_gemm_matrix_cores(T, d, F):
     got = seqmix.moe_experts(h.cuda(), idx.cuda(), wt.cuda(), wgu.cuda(), wd.cuda()).cpu()
     err = (got - want).abs().max() / want.abs().max()
     assert err < 2e-2, float(err)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B", [1, 6, 24], ids=["narrow_blocks", "medium_blocks", "wide_blocks"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_lightning_scan_kernel_widths(B, dtype):
+    """The scan kernel's column-block width follows the batch (8 / 16 / 32
+    columns per workgroup): each against the f32 reference, with unequal
+    sequences, a second step on top of the carried state, and slots in
+    scrambled order."""
+    from loqa_hub_amd.ops import reference as ref
+    from loqa_hub_amd.ops import seqmix
+    g = torch.Generator().manual_seed(B)
+    H, D, Dv = 8, 16, 40
+    n = 2 * H * D + 2 * H * Dv                       # q | k | v | gate columns
+    slots = torch.randperm(B + 3, generator=g)[:B].to(torch.int32)
+    decay = torch.linspace(0.3, 1.0, H)
+    st_ref = torch.zeros(B + 3, H, D, Dv)
+    st_gpu = st_ref.clone().cuda()
+    pos0 = torch.zeros(B, dtype=torch.long)
+    for lens in ([int(x) for x in torch.randint(1, 50, (B,), generator=g)], [1] * B):
+        cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+        T = int(cu[-1])
+        positions = torch.cat([pos0[b] + torch.arange(lens[b]) for b in range(B)]).to(torch.int32)
+        qkv = (torch.randn(T, n, generator=g) * 0.7).to(dtype)
+        want = ref.lightning_scan(qkv, H, D, Dv, st_ref, slots, cu, positions, decay)
+        got = seqmix.lightning_scan(qkv.cuda(), H, D, Dv, st_gpu, slots.cuda(), cu.cuda(),
+                                    positions.cuda(), decay.cuda())
+        scale = want.abs().max()
+        assert (got.cpu() - want).abs().max() / scale < 1e-5
+        pos0 += torch.tensor(lens)
+    assert (st_gpu.cpu() - st_ref).abs().max() / st_ref.abs().max() < 1e-5
