@@ -412,26 +412,39 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_attn2_kernel(LatAttnParams
 }
 
 // out[h, t] from the key splits' (m, l, acc) partials, merged in split order.
+// One wave per (token, head): lane s first turns split s's (m, l) into its
+// weight e^{m_s - M} (M = the largest m, or the sink), then the partial
+// accumulators stream through in split order, four splits in flight.
 template <typename T>
 __global__ __launch_bounds__(64) void latent_combine_kernel(
     const float* __restrict__ ws, const float* __restrict__ sink, T* __restrict__ out, int Tn, int H,
     int R, int S) {
+  __shared__ float fs[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  float M = sink ? sink[h] : -INFINITY;
-  for (int s = 0; s < S; ++s) M = fmaxf(M, ws[(((size_t)s * Tn + t) * H + h) * (R + 2)]);
-  float den = sink ? expf(sink[h] - M) : 0.f;
+  const size_t stride = (size_t)Tn * H * (R + 2);
+  const float* base = ws + ((size_t)t * H + h) * (R + 2);
+  const float ms = lane < S ? base[lane * stride] : -INFINITY;
+  const float ls = lane < S ? base[lane * stride + 1] : 0.f;
+  float M = wave_max(ms);
+  if (sink) M = fmaxf(M, sink[h]);
+  const float f = ms == -INFINITY ? 0.f : expf(ms - M);
+  fs[lane] = f;
+  float den = wave_sum(ls * f);
+  if (sink) den += expf(sink[h] - M);
+  __syncthreads();
   float acc[LAT_MAXR];
 #pragma unroll
   for (int i = 0; i < LAT_MAXR; ++i) acc[i] = 0.f;
+  // unconditional (clamped) loads, so several splits' rows are in flight at once
+#pragma unroll 4
   for (int s = 0; s < S; ++s) {
-    const float* w = ws + (((size_t)s * Tn + t) * H + h) * (R + 2);
-    const float f = w[0] == -INFINITY ? 0.f : expf(w[0] - M);
-    den += w[1] * f;
+    const float* w = base + s * stride + 2;
+    const float fw = fs[s];
+    float v[LAT_MAXR];
 #pragma unroll
-    for (int i = 0; i < LAT_MAXR; ++i) {
-      const int r = lane + 64 * i;
-      if (r < R) acc[i] += w[2 + r] * f;
-    }
+    for (int i = 0; i < LAT_MAXR; ++i) v[i] = w[min(lane + 64 * i, R - 1)];
+#pragma unroll
+    for (int i = 0; i < LAT_MAXR; ++i) acc[i] += v[i] * fw;
   }
   const float inv = den > 0.f ? 1.f / den : 0.f;
 #pragma unroll
@@ -467,6 +480,7 @@ extern "C" int loqa_latent_attention(
   if (T <= 0 || H <= 0) return 0;
   if (R > 64 * LAT_MAXR || R <= 0 || B <= 0) return (int)hipErrorInvalidValue;
   if (num_splits > 1 && !ws) return (int)hipErrorInvalidValue;
+  if (num_splits > 64) return (int)hipErrorInvalidValue;      // one combine lane per split
   LatAttnParams p;
   p.qa = qa; p.qa_st = qa_st; p.qa_sh = qa_sh; p.qr = qr; p.qr_st = qr_st; p.qr_sh = qr_sh;
   p.cache = cache; p.blk = blk; p.cu_q = (const int*)cu_q; p.ctx = (const int*)ctx;

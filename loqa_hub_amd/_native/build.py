@@ -99,8 +99,9 @@ def build(force: bool = False, debug: bool = False, only=None, quiet: bool = Fal
     allk = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.hip")))
     ssrc = [p for p in allk if os.path.basename(p) in SEQMIX_SOURCES]
     ksrc = [p for p in allk if os.path.basename(p) not in SEQMIX_SOURCES]
-    khdr = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.h")))
-    shdr = [p for p in khdr if os.path.basename(p) in ("common.h", "seqmix.h")]
+    allh = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.h")))
+    khdr = [p for p in allh if os.path.basename(p) != "seqmix.h"]
+    shdr = [p for p in allh if os.path.basename(p) in ("common.h", "seqmix.h")]
     rsrc = sorted(glob.glob(os.path.join(CSRC, "runtime", "*.cpp")))
     rhdr = sorted(glob.glob(os.path.join(CSRC, "runtime", "*.h")))
     rflags = [*opt, "-std=c++17", "-D__HIP_PLATFORM_AMD__"]
