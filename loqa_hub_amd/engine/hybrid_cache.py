@@ -2,15 +2,20 @@
 
 Two kinds of per-sequence memory share one sequence table:
 
-* **latent pages**: per caching attention layer a tensor [blocks, BLK, width]
-  (the normalised latent row and the rotated shared key part of each token).
-  The pages of all layers follow ONE block table per sequence, handed out by
-  the same block pool the Llama KV cache uses (native ``BlockPool``);
-* **state slots**: per recurrent layer a tensor [slots + 1, H, D, Dv] f32, one
-  slot per live sequence (the last slot is the write target of padding rows).
-  A slot is taken when a sequence is added and returned with its pages when
-  the sequence is freed; the scan kernel starts a sequence at position 0 from
-  a zero state, so a reused slot needs no clearing.
+* **pages**: per caching attention layer either one tensor [blocks, BLK,
+  width] (latent attention: the normalised latent row and the rotated shared
+  key part of each token) or a key and a value tensor [blocks, BLK, heads x
+  size] (``kv``). The pages of all layers follow ONE block table per sequence,
+  handed out by the same block pool the Llama KV cache uses (native
+  ``BlockPool``);
+* **state slots**: one slot per live sequence (the last slot is the write
+  target of padding rows) in every per-layer state tensor: a recurrent layer's
+  matrix state [slots + 1, H, D, Dv] f32 (``state``), or named f32 rows of any
+  shape [slots + 1, ...] (``rows``: a previous token's activations, the tail
+  of a short convolution). A slot is taken when a sequence is added and
+  returned with its pages when the sequence is freed; the kernels treat the
+  state of a sequence at position 0 as zero, so a reused slot needs no
+  clearing.
 
 Recurrent state cannot be rebuilt from shared prefix pages, so sequences of a
 model with state slots never enter the pool's prefix cache.
@@ -92,7 +97,15 @@ class HybridCache:
                        for li, width in spec["latent"].items()}
         self.state = {li: torch.zeros(max_seqs + 1, H, D, Dv, dtype=torch.float32, device=dev)
                       for li, (H, D, Dv) in spec["state"].items()}
-        self.slots = SlotPool(max_seqs) if self.state else None
+        # key / value pages of plain (uncompressed) attention layers
+        self.kv = {li: (torch.zeros(num_blocks, block_size, kw, dtype=dtype, device=dev),
+                        torch.zeros(num_blocks, block_size, vw, dtype=dtype, device=dev))
+                   for li, (kw, vw) in spec.get("kv", {}).items()}
+        # named per-sequence rows
+        self.rows = {li: {name: torch.zeros(max_seqs + 1, *shape, dtype=torch.float32, device=dev)
+                          for name, shape in named.items()}
+                     for li, named in spec.get("rows", {}).items()}
+        self.slots = SlotPool(max_seqs) if (self.state or self.rows) else None
         self.pool = _SeqPool(make_block_pool(num_blocks, block_size,
                                              require_native=dev.type == "cuda"), self.slots)
 
@@ -107,4 +120,7 @@ class HybridCache:
         return [self.slots.slot(s) for s in seq_ids] + [self.trash_slot] * (B_pad - len(seq_ids))
 
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in (*self.latent.values(), *self.state.values()))
+        ts = [*self.latent.values(), *self.state.values()]
+        ts += [t for pair in self.kv.values() for t in pair]
+        ts += [t for named in self.rows.values() for t in named.values()]
+        return sum(t.numel() * t.element_size() for t in ts)

@@ -257,11 +257,17 @@ class FeedForwardConfig:
     groups: int = 1
     keep: int = 1
     shared_ff: int = 0              # 0: no shared expert
+    # "swiglu": down(silu(gate x) * (up x)); "relu2": down(relu(up x)^2), no gate
+    act: str = "swiglu"
+    # router: "softmax_all" scores every output and weighs by the plain score;
+    # "softmax_top" takes the largest logits (+ bias) and weighs by the softmax
+    # over the chosen ones only
+    router: str = "softmax_all"
 
 
 @dataclass(frozen=True)
 class HybridLayerConfig:
-    kind: str                       # "latent_attention" | "lightning"
+    kind: str                       # "latent_attention" | "lightning" | "attention"
     mixer: object
     mlp: FeedForwardConfig | None
 
@@ -326,3 +332,71 @@ def pipizen_config_from_json(d: dict, name: str = "pipizen") -> PipizenConfig:
                 raise ValueError(f"layer {i}: kv_from must name a latent layer with its own cache")
     return PipizenConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
                          tuple(layers))
+
+
+# --------------------------------------------------------------------------
+# Sodonex: a decoder whose mixer is chunked sigmoid attention (keys double as
+# values, short convolutions on the projections, token shift, per-head output
+# gate), with post-sublayer scalar-gain RMS norms and a mixture of relu^2
+# experts. Every size and constant is taken from config.json or a tensor's shape.
+@dataclass(frozen=True)
+class ChunkAttnConfig:
+    heads: int
+    kv_heads: int
+    dim: int                        # query / key size per head
+    vdim: int                       # value size per head (the values are the keys: == dim)
+    taps: int                       # short causal convolution on q and k
+    chunk: int                      # a query sees earlier keys of its own chunk only
+    scale: float
+    rot: RotaryConfig               # rotate-half layout on the first rot.dims entries
+
+
+@dataclass(frozen=True)
+class SodonexConfig:
+    name: str
+    vocab_size: int
+    d_model: int
+    norm_eps: float
+    residual_mult: float
+    embed_scale: float
+    layers: tuple
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+
+def sodonex_config_from_json(d: dict, name: str = "sodonex") -> SodonexConfig:
+    layers = []
+    for i, L in enumerate(d["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind != "attention":
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        r = m["rot"]
+        mixer = ChunkAttnConfig(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]),
+                                int(m.get("vdim", m["dim"])), int(m["conv"]),
+                                int(m["mask"]["size"]), float(m["scale"]),
+                                RotaryConfig(int(r["dims"]), float(r["base"])))
+        if mixer.heads % mixer.kv_heads:
+            raise ValueError(f"layer {i}: {mixer.heads} heads do not split over "
+                             f"{mixer.kv_heads} key/value heads")
+        if mixer.vdim != mixer.dim:
+            raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim")
+        if mixer.rot.dims % 2 or not 0 <= mixer.rot.dims <= mixer.dim:
+            raise ValueError(f"layer {i}: rot.dims {mixer.rot.dims} does not fit a head of {mixer.dim}")
+        if mixer.taps < 1 or mixer.chunk < 1:
+            raise ValueError(f"layer {i}: conv taps and mask size must be positive")
+        f = L.get("mlp")
+        if not f:
+            mlp = None
+        elif f["kind"] == "moe":
+            r = f["router"]
+            mlp = FeedForwardConfig("moe", int(f["expert"]["ff"]), int(r["experts"]), 0,
+                                    int(r["top"]), act="relu2", router="softmax_top")
+            if not 0 < mlp.top <= mlp.experts:
+                raise ValueError(f"layer {i}: top {mlp.top} of {mlp.experts} experts")
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(HybridLayerConfig(kind, mixer, mlp))
+    return SodonexConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]),
+                         float(d["residual_mult"]), float(d["embedding"]["scale"]), tuple(layers))

@@ -1,6 +1,7 @@
 """Language-model families the LLM engine can serve, chosen by a checkpoint's
-config.json: the Llama family (Hugging Face naming) and the hybrid Pipizen
-design (its own naming, ``"architecture": "Pipizen"``). A family knows how to
+config.json: the Llama family (Hugging Face naming) and the designs with their
+own naming, told apart by ``"architecture"``: the hybrid Pipizen (latent /
+lightning mixers) and Sodonex (chunked sigmoid attention with row state). A family knows how to
 read its config, load or seed its weights and build its step function; the
 engine, the scheduler and the command line go through this table only.
 """
@@ -11,8 +12,8 @@ from typing import Callable
 
 import torch
 
-from .configs import (LlamaConfig, PipizenConfig, checkpoint_config, llama_config_from_hf,
-                      pipizen_config_from_json)
+from .configs import (LlamaConfig, PipizenConfig, SodonexConfig, checkpoint_config,
+                      llama_config_from_hf, pipizen_config_from_json, sodonex_config_from_json)
 
 
 @dataclass(frozen=True)
@@ -21,11 +22,15 @@ class Family:
     config_cls: type
     matches: Callable[[dict], bool]
     config_from_json: Callable[[dict, str], object]
-    hybrid: bool            # latent pages + state slots (engine/hybrid_cache.py)
+    hybrid: bool            # pages + state slots (engine/hybrid_cache.py)
 
 
 def _is_pipizen(d: dict) -> bool:
     return str(d.get("architecture", "")).lower() == "pipizen"
+
+
+def _is_sodonex(d: dict) -> bool:
+    return str(d.get("architecture", "")).lower() == "sodonex"
 
 
 def _is_llama(d: dict) -> bool:
@@ -35,6 +40,7 @@ def _is_llama(d: dict) -> bool:
 
 FAMILIES = (
     Family("pipizen", PipizenConfig, _is_pipizen, pipizen_config_from_json, True),
+    Family("sodonex", SodonexConfig, _is_sodonex, sodonex_config_from_json, True),
     Family("llama", LlamaConfig, _is_llama, llama_config_from_hf, False),
 )
 
@@ -73,6 +79,8 @@ def load_lm_weights(cfg, path: str, device, *, dtype=torch.bfloat16, tp=None,
         return loader.load_llama(cfg, path, device, tp)
     if tp is not None and tp.world > 1:
         raise ValueError(f"{fam.name}: tensor parallel serving is not available")
+    if fam.name == "sodonex":
+        return loader.load_sodonex(cfg, path, device, dtype, max_positions)
     return loader.load_pipizen(cfg, path, device, dtype, max_positions)
 
 
@@ -82,6 +90,9 @@ def random_lm_weights(cfg, device, *, seed: int = 0, dtype=torch.bfloat16, tp=No
     if fam.name == "llama":
         from .llama import LlamaWeights
         return LlamaWeights(cfg, device, seed=seed, tp=tp, compact=compact)
+    if fam.name == "sodonex":
+        from .sodonex import SodonexWeights
+        return SodonexWeights.random(cfg, device, seed, dtype, max_positions)
     from .pipizen import PipizenWeights
     return PipizenWeights.random(cfg, device, seed, dtype, max_positions)
 
@@ -90,5 +101,8 @@ def build_model(weights):
     from .llama import LlamaModel, LlamaWeights
     if isinstance(weights, LlamaWeights):
         return LlamaModel(weights)
+    from .sodonex import SodonexModel, SodonexWeights
+    if isinstance(weights, SodonexWeights):
+        return SodonexModel(weights)
     from .pipizen import PipizenModel
     return PipizenModel(weights)

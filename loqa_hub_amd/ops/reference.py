@@ -728,12 +728,19 @@ def gated_rmsnorm(o, w, gate, eps: float, out_dtype):
     return (y * torch.sigmoid(gate.float())).to(out_dtype)
 
 
-def moe_route(z, correction, n_groups: int, keep: int, top: int):
-    """z f32 [T, E] router logits -> (expert index int32 [T, top], weight f32
-    [T, top]). Scores are softmax(z); experts are chosen by score + correction
-    among the ``keep`` best of ``n_groups`` equal groups of neighbours (a
-    group's rank is its best choice score); the weights are the plain scores."""
-    s = torch.softmax(z.float(), dim=-1)
+def moe_route(z, correction, n_groups: int, keep: int, top: int, bias=None,
+              top_softmax: bool = False):
+    """z f32 [T, E] router logits (+ ``bias`` [E]) -> (expert index int32 [T, top],
+    weight f32 [T, top]). Default: scores are softmax(z); experts are chosen by
+    score + correction among the ``keep`` best of ``n_groups`` equal groups of
+    neighbours (a group's rank is its best choice score); the weights are the
+    plain scores. ``top_softmax``: the ``top`` largest logits are chosen and the
+    weights are the softmax over the chosen logits only."""
+    z = z.float() if bias is None else z.float() + bias.float()
+    if top_softmax:
+        best = z.topk(top, dim=-1)
+        return best.indices.to(torch.int32), torch.softmax(best.values, dim=-1)
+    s = torch.softmax(z, dim=-1)
     choice = s if correction is None else s + correction.float()
     if n_groups > 1 and keep < n_groups:
         T, E = s.shape
@@ -746,14 +753,16 @@ def moe_route(z, correction, n_groups: int, keep: int, top: int):
     return idx.to(torch.int32), s.gather(1, idx)
 
 
-def moe_experts(h, idx, wt, w_gate_up, w_down, out_dtype):
-    """Weighted sum of each token's chosen experts: expert e < E is the gated
-    feed-forward (w_gate_up [E, 2F, d] = gate | up rows, w_down [E, d, F]);
-    an index >= E is an identity expert (its output is h). Returns f32 [T, d];
-    the expert outputs are rounded to ``out_dtype`` first, as GEMM outputs."""
+def moe_experts(h, idx, wt, w_gate_up, w_down, out_dtype, gated: bool = True):
+    """Weighted sum of each token's chosen experts: expert e < E is a
+    feed-forward - gated: down(silu(gate x) * (up x)) with w_gate_up [E, 2F, d]
+    = gate | up rows; not gated: down(relu(up x)^2) with w_gate_up [E, F, d] -
+    and w_down [E, d, F]; an index >= E is an identity expert (its output is
+    h). Returns f32 [T, d]; the expert outputs are rounded to ``out_dtype``
+    first, as GEMM outputs."""
     T, d = h.shape
     E = w_gate_up.shape[0]
-    F = w_gate_up.shape[1] // 2
+    F = w_gate_up.shape[1] // 2 if gated else w_gate_up.shape[1]
     out = torch.zeros(T, d, dtype=torch.float32, device=h.device)
     for k in range(idx.shape[1]):
         e = idx[:, k].long()
@@ -763,7 +772,162 @@ def moe_experts(h, idx, wt, w_gate_up, w_down, out_dtype):
             rows = (e == ee).nonzero()[:, 0]
             x = h[rows].to(out_dtype)
             gu = torch.nn.functional.linear(x, w_gate_up[ee])
-            a = (torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()).to(out_dtype)
+            if gated:
+                a = (torch.nn.functional.silu(gu[:, :F].float()) * gu[:, F:].float()).to(out_dtype)
+            else:
+                a = torch.relu(gu.float()).pow(2).to(out_dtype)
             y = torch.nn.functional.linear(a, w_down[ee])
             out[rows] += wt[rows, k:k + 1] * y.float()
     return out
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of decoders with per-sequence row state (models/sodonex.py):
+# token shift, short causal convolutions with a carried tail, whole-projection
+# RMS norm + rotate-half rotary + paged K/V append, chunked sigmoid attention
+# with a per-head output gate, and a scalar-gain RMS norm on the residual step.
+def rope_table_half(dims: int, max_pos: int, base: float, device=None) -> torch.Tensor:
+    """[max_pos, dims/2, 2] f32 (cos, sin) for the rotate-half layout (entry i
+    turns with entry i + dims/2 by position * base^(-2i/dims)); angles in f64."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / max(dims, 1))
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None, :]
+    return torch.stack([ang.cos(), ang.sin()], dim=-1).float().to(device)
+
+
+def token_shift(x, mu, prev, state_slots, cu_q, positions, out_dtype):
+    """h_t = x_t + (x_{t-1} - x_t) * mu; the row before a feed's first token
+    is the sequence's saved row ``prev[slot]`` (zeros at position 0)."""
+    xf = x.float()
+    h = torch.empty_like(xf)
+    cu = cu_q.tolist()
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        first = torch.zeros_like(xf[0]) if int(positions[q0]) == 0 else prev[int(state_slots[b])]
+        before = torch.cat([first[None], xf[q0:q1 - 1]])
+        h[q0:q1] = xf[q0:q1] + (before - xf[q0:q1]) * mu.float()
+    return h.to(out_dtype)
+
+
+def seq_state_save(x, u, prev, tail, state_slots, cu_q, positions):
+    """After a step: prev[slot] = the feed's last row of x; tail[slot]
+    [taps - 1, C] = the last taps - 1 rows of the projections u[:, :C] (older
+    rows move up when the feed is shorter; zeros before the sequence's start)."""
+    cu = cu_q.tolist()
+    keep, C = tail.shape[1], tail.shape[2]
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        slot = int(state_slots[b])
+        if prev is not None:
+            prev[slot] = x[q1 - 1].float()
+        if keep:
+            old = torch.zeros_like(tail[slot]) if int(positions[q0]) == 0 else tail[slot].clone()
+            rows = torch.cat([old, u[q0:q1, :C].float()])
+            tail[slot] = rows[-keep:]
+
+
+def conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm, k_norm, eps: float,
+                          cos_sin, dims: int, H: int, G: int, D: int, k_cache, v_cache, slots,
+                          out_dtype):
+    """u [T, >= (H + G) D]: the projected q | k rows. Causal per-channel
+    convolution (weights conv_w [(H + G) D, taps], the rows before the feed from
+    ``tail[slot]``), then: v = the convolved k; q and k each RMS-normed over the
+    whole projection (weights q_norm / k_norm), rotated (rotate-half, the first
+    ``dims`` entries of every head); k and v go to the paged caches
+    [blocks, BLK, G D] at ``slots``; returns q [T, H D]."""
+    T = u.shape[0]
+    C, taps = conv_w.shape
+    Cq = H * D
+    cu = cu_q.tolist()
+    y = torch.zeros(T, C, dtype=torch.float32, device=u.device)
+    w = conv_w.float()
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        if taps > 1:
+            old = torch.zeros_like(tail[0]) if int(positions[q0]) == 0 else \
+                tail[int(state_slots[b])]
+            rows = torch.cat([old.float(), u[q0:q1, :C].float()])
+        else:
+            rows = u[q0:q1, :C].float()
+        n = q1 - q0
+        for j in range(taps):
+            y[q0:q1] += rows[j:j + n] * w[:, j]
+    yq, yk = y[:, :Cq], y[:, Cq:]
+    v = yk.to(v_cache.dtype)
+    q = yq * torch.rsqrt(yq.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()
+    k = yk * torch.rsqrt(yk.pow(2).mean(-1, keepdim=True) + eps) * k_norm.float()
+    cs = cos_sin[positions[:T].long()]                          # [T, dims/2, 2]
+
+    def turn(x, heads):
+        x = x.view(T, heads, D).clone()
+        half = dims // 2
+        a, bb = x[..., :half].clone(), x[..., half:dims].clone()
+        c, s = cs[:, None, :, 0], cs[:, None, :, 1]
+        x[..., :half] = a * c - bb * s
+        x[..., half:dims] = bb * c + a * s
+        return x.view(T, heads * D)
+    if dims:
+        q, k = turn(q, H), turn(k, G)
+    sl = slots[:T].long()
+    ok = sl >= 0
+    blk = k_cache.shape[1]
+    k_cache[(sl // blk)[ok], (sl % blk)[ok]] = k.to(k_cache.dtype)[ok]
+    v_cache[(sl // blk)[ok], (sl % blk)[ok]] = v[ok]
+    return q.to(out_dtype)
+
+
+def sigmoid_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions, head_bias,
+                      gate, scale: float, chunk: int, H: int, G: int, D: int, out_dtype):
+    """q [T, H D] against the paged caches [blocks, BLK, G D]: a query at
+    position p sees keys j <= p (with ``chunk`` > 0 only those of its own
+    chunk, j // chunk == p // chunk); a visible key weighs
+    sigmoid(q . k * scale + head_bias[h]), not normalised over keys; head h's
+    output is multiplied by sigmoid(gate[t, h]). Returns [T, H D]."""
+    T = q.shape[0]
+    blk = k_cache.shape[1]
+    rep = H // G
+    cu = cu_q.tolist()
+    out = torch.zeros(T, H, D, dtype=torch.float32, device=q.device)
+    qf = q.float().view(T, H, D)
+    for b in range(len(cu) - 1):
+        q0, q1 = cu[b], cu[b + 1]
+        if q1 == q0:
+            continue
+        L = int(ctx_lens[b])
+        idx = torch.arange(L, device=q.device)
+        tab = block_tables[b].long()
+        kk = k_cache[tab[idx // blk], idx % blk].float().view(L, G, D)
+        vv = v_cache[tab[idx // blk], idx % blk].float().view(L, G, D)
+        qpos = positions[q0:q1].long()
+        seen = idx[None, :] <= qpos[:, None]
+        if chunk > 0:
+            seen &= (idx[None, :] // chunk) == (qpos[:, None] // chunk)
+        for h in range(H):
+            s = qf[q0:q1, h] @ kk[:, h // rep].T * scale + head_bias[h].float()
+            w = torch.sigmoid(s) * seen
+            out[q0:q1, h] = w @ vv[:, h // rep]
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[:, :, None]
+    return out.view(T, H * D).to(out_dtype)
+
+
+def scalar_rms_add(resid, y, g: float, eps: float, mult: float, out_dtype):
+    """resid (f32, in place) += mult * y / rms(y) * g; returns resid in
+    ``out_dtype`` (None: nothing)."""
+    yf = y.float()
+    resid.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * (g * mult))
+    return None if out_dtype is None else resid.to(out_dtype)
+
+
+def scalar_rms_norm(x, g: float, eps: float, row_idx=None):
+    """f32 rows of x / rms(x) * g (``row_idx`` gathers rows first)."""
+    if row_idx is not None:
+        x = x.index_select(0, row_idx.long())
+    xf = x.float()
+    return xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * g

@@ -292,44 +292,50 @@ def silu_mul_any(x: torch.Tensor) -> torch.Tensor:
 
 
 def moe_route(z: torch.Tensor, correction: torch.Tensor | None, n_groups: int, keep: int,
-              top: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """Router decisions from f32 logits z [T, E]: softmax scores, choice by
-    score + ``correction`` limited to the ``keep`` best of ``n_groups`` groups of
-    neighbouring experts, weights = the plain scores (not renormalised).
+              top: int, bias: torch.Tensor | None = None, top_softmax: bool = False
+              ) -> tuple[torch.Tensor, torch.Tensor]:
+    """Router decisions from f32 logits z [T, E] (+ ``bias`` [E]). Default:
+    softmax scores, choice by score + ``correction`` limited to the ``keep``
+    best of ``n_groups`` groups of neighbouring experts, weights = the plain
+    scores (not renormalised). ``top_softmax``: the ``top`` largest logits are
+    chosen and weighed by the softmax over the chosen logits only.
     Returns (idx int32 [T, top], weight f32 [T, top])."""
     if not z.is_cuda:
-        return ref.moe_route(z, correction, n_groups, keep, top)
+        return ref.moe_route(z, correction, n_groups, keep, top, bias, top_softmax)
     _f32c(z, "z")
     T, E = z.shape
     assert E % max(1, n_groups) == 0 and 0 < top <= E and E <= 1024
-    if correction is not None:
-        _f32c(correction, "correction")
-        assert correction.numel() == E
+    for v, name in ((correction, "correction"), (bias, "bias")):
+        if v is not None:
+            _f32c(v, name)
+            assert v.numel() == E
     idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
     wt = torch.empty(T, top, dtype=torch.float32, device=z.device)
     if T:
-        check(kernels().loqa_moe_route(ptr(z), ptr(correction), E, max(1, n_groups),
-                                       min(keep, max(1, n_groups)), top, ptr(idx), ptr(wt), T,
-                                       stream_ptr(z)), "moe_route")
+        check(kernels().loqa_moe_route(ptr(z), ptr(correction), ptr(bias), int(top_softmax), E,
+                                       max(1, n_groups), min(keep, max(1, n_groups)), top, ptr(idx),
+                                       ptr(wt), T, stream_ptr(z)), "moe_route")
     return idx, wt
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor, w_gate_up: torch.Tensor,
-                w_down: torch.Tensor) -> torch.Tensor:
+                w_down: torch.Tensor, gated: bool = True) -> torch.Tensor:
     """Weighted sum of every token's chosen experts, f32 [T, d]. Experts below
-    E = w_gate_up.shape[0] are gated feed-forwards (w_gate_up [E, 2F, d] with
-    gate rows then up rows, w_down [E, d, F]); an index >= E is an identity
-    expert. On the GPU: a device-side plan (tokens grouped by expert, no host
-    round trip), a grouped gate|up GEMM with the SwiGLU epilogue, a grouped
-    down GEMM, and a combine launch that applies the weights in f32."""
+    E = w_gate_up.shape[0] are feed-forwards: gated (w_gate_up [E, 2F, d] with
+    gate rows then up rows, SwiGLU) or not (w_gate_up [E, F, d], the square of
+    relu), w_down [E, d, F]; an index >= E is an identity expert. On the GPU: a
+    device-side plan (tokens grouped by expert, no host round trip), a grouped
+    up GEMM with the activation as its epilogue, a grouped down GEMM, and a
+    combine launch that applies the weights in f32."""
     if not h.is_cuda:
-        return ref.moe_experts(h, idx, wt, w_gate_up, w_down, h.dtype)
+        return ref.moe_experts(h, idx, wt, w_gate_up, w_down, h.dtype, gated)
     T, d = h.shape
     E, F2, _ = w_gate_up.shape
-    F = F2 // 2
+    F = F2 // 2 if gated else F2
     top = idx.shape[1]
     assert h.is_contiguous() and w_gate_up.is_contiguous() and w_down.is_contiguous()
     assert w_gate_up.dtype == h.dtype == w_down.dtype and w_down.shape == (E, d, F)
+    assert w_gate_up.shape[2] == d
     _i32c(idx, "idx"); _f32c(wt, "wt")
     dev = h.device
     P = T * top
@@ -343,10 +349,195 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor, w_gate_up:
     y = torch.empty(P, d, dtype=h.dtype, device=dev)
     k, st = kernels(), stream_ptr(h)
     check(k.loqa_moe_plan(ptr(idx), P, E, ptr(plan), st), "moe_plan")
-    check(k.loqa_moe_grouped_gemm(ptr(h), _dt(h), ptr(w_gate_up), ptr(plan), P, E, top, d, F, 1,
-                                  ptr(act), st), "moe_gate_up")
+    check(k.loqa_moe_grouped_gemm(ptr(h), _dt(h), ptr(w_gate_up), ptr(plan), P, E, top, d, F,
+                                  1 if gated else 2, ptr(act), st), "moe_up")
     check(k.loqa_moe_grouped_gemm(ptr(act), _dt(h), ptr(w_down), ptr(plan), P, E, top, F, d, 0,
                                   ptr(y), st), "moe_down")
     check(k.loqa_moe_combine(ptr(h), ptr(y), _dt(h), ptr(idx), ptr(wt), ptr(plan), T, top, E, d,
                              ptr(out), st), "moe_combine")
     return out
+
+
+# ---------------------------------------------------------------------------
+# Per-sequence row state (token shift, convolution tails), chunked sigmoid
+# attention over paged K/V, scalar-gain RMS norm on the residual step
+# (csrc/kernels/seq_rows.hip, attn_sigmoid.hip, norm_scalar.hip)
+def rope_table_half(dims: int, max_pos: int, base: float, device=None) -> torch.Tensor:
+    """(cos, sin) table of the rotate-half rotary layout, built once at load time."""
+    return ref.rope_table_half(dims, max_pos, base, device)
+
+
+def _seq_args(state_slots, cu_q, positions, T):
+    _i32c(state_slots, "state_slots"); _i32c(cu_q, "cu_q"); _i32c(positions, "positions")
+    B = state_slots.numel()
+    assert cu_q.numel() == B + 1 and positions.numel() >= T
+    return B
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, prev: torch.Tensor, state_slots: torch.Tensor,
+                cu_q: torch.Tensor, positions: torch.Tensor, out_dtype) -> torch.Tensor:
+    """h_t = x_t + (x_{t-1} - x_t) * mu over a flat token batch x f32 [T, d];
+    the row before a feed's first token is ``prev[slot]`` f32 [slots, d] (zeros
+    when the feed starts at position 0). ``prev`` is not written here
+    (:func:`seq_state_save` does, once every reader of the step is done)."""
+    if not x.is_cuda:
+        return ref.token_shift(x, mu, prev, state_slots, cu_q, positions, out_dtype)
+    _f32c(x, "x"); _f32c(mu, "mu"); _f32c(prev, "prev")
+    T, d = x.shape
+    assert mu.numel() == d and prev.shape[1] == d
+    B = _seq_args(state_slots, cu_q, positions, T)
+    h = torch.empty(T, d, dtype=out_dtype, device=x.device)
+    if T:
+        check(kernels().loqa_token_shift(ptr(x), ptr(mu), ptr(prev), prev.shape[0], ptr(state_slots),
+                                         ptr(cu_q), ptr(positions), B, T, d, ptr(h), _dt(h),
+                                         stream_ptr(x)), "token_shift")
+    return h
+
+
+def seq_state_save(x: torch.Tensor | None, u: torch.Tensor, prev: torch.Tensor | None,
+                   tail: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+                   positions: torch.Tensor) -> None:
+    """The step's row state: prev[slot] = the last row of each feed of x f32
+    [T, d]; tail[slot] f32 [taps - 1, C] = the last taps - 1 rows of the
+    projections u[:, :C] (older rows move up under a shorter feed)."""
+    if not u.is_cuda:
+        return ref.seq_state_save(x, u, prev, tail, state_slots, cu_q, positions)
+    T = u.shape[0]
+    _f32c(tail, "tail")
+    keep, C = tail.shape[1], tail.shape[2]
+    assert u.stride(1) == 1 and u.shape[1] >= C
+    d = 0
+    if prev is not None:
+        _f32c(x, "x"); _f32c(prev, "prev")
+        d = x.shape[1]
+        assert prev.shape == (tail.shape[0], d) and x.shape[0] == T
+    B = _seq_args(state_slots, cu_q, positions, T)
+    if T:
+        check(kernels().loqa_seq_state_save(ptr(x), d, ptr(u), _dt(u), u.stride(0), ptr(prev),
+                                            ptr(tail), tail.shape[0], keep, C, ptr(state_slots),
+                                            ptr(cu_q), ptr(positions), B, stream_ptr(u)),
+              "seq_state_save")
+
+
+def conv_norm_rope_append(u: torch.Tensor, conv_w: torch.Tensor, tail: torch.Tensor,
+                          state_slots: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor,
+                          q_norm: torch.Tensor, k_norm: torch.Tensor, eps: float,
+                          cos_sin: torch.Tensor, dims: int, H: int, G: int, D: int,
+                          k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor,
+                          out_dtype) -> torch.Tensor:
+    """One launch between the q | k projection and attention: short causal
+    convolution per channel (f32 weights conv_w [(H + G) D, taps]; the rows
+    before a feed come from ``tail[slot]``), v = the convolved k, RMS norm of q
+    and of k over the whole projection, rotate-half rotary on the first
+    ``dims`` entries of every head, k and v into the paged caches
+    [blocks, BLK, G D]; returns q [T, H D]."""
+    if not u.is_cuda:
+        return ref.conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm,
+                                         k_norm, eps, cos_sin, dims, H, G, D, k_cache, v_cache,
+                                         slots, out_dtype)
+    T = u.shape[0]
+    C, taps = conv_w.shape
+    assert C == (H + G) * D and u.stride(1) == 1 and u.shape[1] >= C
+    _f32c(conv_w, "conv_w"); _f32c(tail, "tail"); _f32c(q_norm, "q_norm"); _f32c(k_norm, "k_norm")
+    _f32c(cos_sin, "cos_sin"); _i32c(slots, "slots")
+    assert tail.shape[1:] == (taps - 1, C) and q_norm.numel() == H * D and k_norm.numel() == G * D
+    assert dims % 2 == 0 and dims <= D and (dims == 0 or cos_sin.shape[1] * 2 == dims)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    assert k_cache.shape[2] == G * D and k_cache.dtype == v_cache.dtype == out_dtype
+    assert slots.numel() >= T
+    B = _seq_args(state_slots, cu_q, positions, T)
+    q = torch.empty(T, H * D, dtype=out_dtype, device=u.device)
+    if T:
+        check(kernels().loqa_conv_norm_rope_append(
+            ptr(u), _dt(u), u.stride(0), ptr(conv_w), taps, ptr(tail), tail.shape[0],
+            ptr(state_slots), ptr(cu_q), ptr(positions), B, T, ptr(q_norm), ptr(k_norm), eps,
+            ptr(cos_sin), cos_sin.shape[0], dims, H, G, D, ptr(k_cache), ptr(v_cache),
+            k_cache.shape[1], k_cache.shape[0], ptr(slots), ptr(q), _dt(q), stream_ptr(u)),
+            "conv_norm_rope_append")
+    return q
+
+
+SIGMOID_MFMA_D = (64, 128)        # head sizes the matrix-core form is built for
+
+
+def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      cu_q: torch.Tensor, ctx_lens: torch.Tensor, block_tables: torch.Tensor,
+                      positions: torch.Tensor, head_bias: torch.Tensor, gate: torch.Tensor | None,
+                      scale: float, chunk: int, H: int, G: int, D: int, max_q: int = 0,
+                      matrix_cores: bool | None = None) -> torch.Tensor:
+    """Attention without softmax over paged K/V [blocks, BLK, G D]: a query at
+    position p sees keys j <= p - with ``chunk`` > 0 only those of its own chunk
+    (j // chunk == p // chunk, counted from the sequence's start) - and a
+    visible key weighs sigmoid(q . k * scale + head_bias[h]) (f32, not
+    normalised over keys). Head h's output is multiplied by sigmoid(gate[t, h])
+    (``gate`` [T, H], may be a column slice). q [T, H D] -> [T, H D]. Prompt
+    portions, decode tokens and mixed batches take the same launch; every
+    output sums its keys in ascending position order whatever the batch."""
+    if not q.is_cuda:
+        return ref.sigmoid_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions,
+                                     head_bias, gate, scale, chunk, H, G, D, q.dtype)
+    T = q.shape[0]
+    assert q.is_contiguous() and q.shape[1] == H * D and H % G == 0
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    assert k_cache.shape[2] == G * D and k_cache.dtype == v_cache.dtype == q.dtype
+    _i32c(cu_q, "cu_q"); _i32c(ctx_lens, "ctx_lens"); _i32c(block_tables, "block_tables")
+    _i32c(positions, "positions"); _f32c(head_bias, "head_bias")
+    B = ctx_lens.numel()
+    assert cu_q.numel() == B + 1 and block_tables.shape[0] == B and positions.numel() >= T
+    assert head_bias.numel() == H
+    gs = 0
+    if gate is not None:
+        assert gate.shape == (T, H) and gate.stride(1) == 1 and gate.dtype == q.dtype
+        gs = gate.stride(0)
+    o = torch.empty(T, H * D, dtype=q.dtype, device=q.device)
+    if matrix_cores is None:
+        matrix_cores = max_q >= 16
+    mfma = bool(matrix_cores) and q.dtype == torch.bfloat16 and D in SIGMOID_MFMA_D
+    if T:
+        check(kernels().loqa_sigmoid_attention(
+            ptr(q), _dt(q), ptr(k_cache), ptr(v_cache), k_cache.shape[1], k_cache.shape[0],
+            ptr(cu_q), ptr(ctx_lens), ptr(block_tables), block_tables.shape[1], ptr(positions),
+            ptr(head_bias), ptr(gate), gs, float(scale), int(chunk), B, T, H, G, D, int(max_q),
+            int(mfma), ptr(o), stream_ptr(q)), "sigmoid_attention")
+    return o
+
+
+def scalar_rms_add(resid: torch.Tensor, y: torch.Tensor, g: float, eps: float, mult: float,
+                   out_dtype=None) -> torch.Tensor | None:
+    """The residual step with a norm on the sublayer's output only: resid (f32,
+    in place) += mult * y / rms(y) * g with ONE gain g for all coordinates; the
+    same launch returns resid in ``out_dtype`` for the next sublayer's GEMMs
+    (None: nothing; float32: resid itself)."""
+    if not resid.is_cuda:
+        ref.scalar_rms_add(resid, y, g, eps, mult, None)
+        if out_dtype is None:
+            return None
+        return resid if out_dtype == torch.float32 else resid.to(out_dtype)
+    _f32c(resid, "resid")
+    assert y.shape == resid.shape and y.is_contiguous()
+    rows, d = resid.shape
+    copy = out_dtype is not None and out_dtype != torch.float32
+    h = torch.empty(rows, d, dtype=out_dtype, device=resid.device) if copy else None
+    if rows:
+        check(kernels().loqa_scalar_rms_add(ptr(resid), ptr(y), _dt(y), float(g) * float(mult),
+                                            float(eps), ptr(h), rows, d, stream_ptr(resid)),
+              "scalar_rms_add")
+    return h if copy else (resid if out_dtype == torch.float32 else None)
+
+
+def scalar_rms_norm(x: torch.Tensor, g: float, eps: float, row_idx: torch.Tensor | None = None
+                    ) -> torch.Tensor:
+    """f32 rows of x / rms(x) * g for x f32 [rows, d]; ``row_idx`` (int64)
+    gathers rows in the same launch."""
+    if not x.is_cuda:
+        return ref.scalar_rms_norm(x, g, eps, row_idx)
+    _f32c(x, "x")
+    d = x.shape[1]
+    rows = x.shape[0] if row_idx is None else row_idx.numel()
+    if row_idx is not None:
+        assert row_idx.dtype == torch.int64 and row_idx.is_contiguous()
+    y = torch.empty(rows, d, dtype=torch.float32, device=x.device)
+    if rows:
+        check(kernels().loqa_scalar_rms_norm(ptr(x), ptr(row_idx), float(g), float(eps), ptr(y), rows,
+                                             d, stream_ptr(x)), "scalar_rms_norm")
+    return y
