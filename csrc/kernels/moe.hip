@@ -5,7 +5,9 @@
 //   outputs; choice = score + correction; router outputs form `groups` equal
 //   groups of neighbours, a group ranks by its best choice score and only the
 //   `keep` best groups stay eligible (the others count as -inf); the `top`
-//   best eligible choices are taken; the weights are the plain scores.
+//   best eligible choices are taken; the weights are the plain scores. With
+//   `top_softmax` the choice is by the logit itself (+ bias) and the weights
+//   are the softmax over the chosen logits only.
 // moe_plan_kernel (one workgroup): (token, k) pairs bucketed by expert without
 //   a host round trip: offsets[E + 2], perm[P] (pair ids in expert order; the
 //   identity bucket E last), pos[P] (where each pair sits).
@@ -13,7 +15,8 @@
 //   f32 accumulation over K in ascending order for every output element (so a
 //   pair's result does not depend on which other pairs share its tile). Mode
 //   1 gathers A rows by token and applies the SwiGLU epilogue to the (gate,
-//   up) weight row pairs; mode 0 reads the sorted activation rows.
+//   up) weight row pairs; mode 2 gathers A rows by token and squares the relu
+//   of a single (up) weight set; mode 0 reads the sorted activation rows.
 // moe_combine_kernel: out[t] = sum_k weight * (expert output | the input
 //   itself for an identity expert), f32.
 #include "seqmix.h"
@@ -30,23 +33,29 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 }
 
 __global__ __launch_bounds__(64) void moe_route_kernel(
-    const float* __restrict__ z, const float* __restrict__ corr, int E, int G, int keep, int top,
-    int* __restrict__ idx, float* __restrict__ wt) {
+    const float* __restrict__ z, const float* __restrict__ corr, const float* __restrict__ bias,
+    int top_softmax, int E, int G, int keep, int top, int* __restrict__ idx,
+    float* __restrict__ wt) {
   __shared__ float sc[MOE_MAX_E], ch[MOE_MAX_E], gs[MOE_MAX_E];
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (size_t)t * E;
   float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+  for (int e = lane; e < E; e += 64) {
+    const float v = bias ? zr[e] + bias[e] : zr[e];
+    gs[e] = v;                                  // the logit with its bias
+    mx = fmaxf(mx, v);
+  }
   mx = wave_max(mx);
   float sum = 0.f;
   for (int e = lane; e < E; e += 64) {
-    const float v = expf(zr[e] - mx);
+    const float v = expf(gs[e] - mx);
     sc[e] = v;
     sum += v;
   }
   sum = wave_sum(sum);
   const float inv = 1.f / sum;
   for (int e = lane; e < E; e += 64) {
+    if (top_softmax) { ch[e] = gs[e]; continue; }      // scores stay unnormalised: see below
     const float s = sc[e] * inv;
     sc[e] = s;
     ch[e] = corr ? s + corr[e] : s;
@@ -92,6 +101,13 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
     }
     __syncthreads();
   }
+  if (top_softmax && lane == 0) {
+    // softmax over the chosen logits: exp(z - max) of the chosen ones over their sum
+    float tot = 0.f;
+    for (int k = 0; k < top; ++k) tot += wt[(size_t)t * top + k];
+    const float r = 1.f / tot;
+    for (int k = 0; k < top; ++k) wt[(size_t)t * top + k] *= r;
+  }
 }
 
 __global__ __launch_bounds__(256) void moe_plan_kernel(const int* __restrict__ idx, int P, int E,
@@ -129,10 +145,14 @@ __global__ __launch_bounds__(256) void moe_plan_kernel(const int* __restrict__ i
 #define GG_T 64
 #define GG_K 16
 
-template <typename T, int SWIGLU>
+__device__ __forceinline__ float relu2_f(float z) { const float r = fmaxf(z, 0.f); return r * r; }
+
+template <typename T, int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(
     const T* __restrict__ A, const T* __restrict__ Wt, const int* __restrict__ plan, int P, int E,
     int top, int K, int N, T* __restrict__ out) {
+  constexpr int SWIGLU = MODE == 1;
+  constexpr bool GATHER = MODE != 0;
   __shared__ float As[GG_K][GG_T + 1], Bs[GG_K][GG_T + 1], Bu[SWIGLU ? GG_K : 1][GG_T + 1];
   const int* offsets = plan;
   const int* perm = plan + E + 2;
@@ -161,7 +181,7 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(
       float a = 0.f, b = 0.f, u = 0.f;
       if (k0 + kk < K) {
         if (r0 + r < r1) {
-          const size_t src = SWIGLU ? (size_t)(perm[r0 + r] / top) : (size_t)(r0 + r);
+          const size_t src = GATHER ? (size_t)(perm[r0 + r] / top) : (size_t)(r0 + r);
           a = Act<T>::ld(A + src * K + k0 + kk);
         }
         if (n0 + r < N) {
@@ -200,7 +220,8 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n < N)
-        Act<T>::st(out + (size_t)r * N + n, SWIGLU ? silu_f(acc[i][j]) * accu[i][j] : acc[i][j]);
+        Act<T>::st(out + (size_t)r * N + n, SWIGLU ? silu_f(acc[i][j]) * accu[i][j]
+                                                   : MODE == 2 ? relu2_f(acc[i][j]) : acc[i][j]);
     }
   }
 }
@@ -214,10 +235,12 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_kernel(
 // the 16 matching up-rows for SwiGLU) against all 64 rows, so the row fragments
 // are shared through L1. An accumulator lane holds 4 consecutive features of
 // one token row. Per output element the sum over K has a fixed order.
-template <int SWIGLU>
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wt, const int* __restrict__ plan, int P,
     int E, int top, int K, int N, bf16_t* __restrict__ out) {
+  constexpr int SWIGLU = MODE == 1;
+  constexpr bool GATHER = MODE != 0;
   const int* offsets = plan;
   const int* perm = plan + E + 2;
   int tile = blockIdx.x, e = 0, r0 = 0, r1 = 0;
@@ -241,7 +264,7 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int r = min(r0 + 16 * j + fr, r1 - 1);
-    const size_t src = SWIGLU ? (size_t)(perm[r] / top) : (size_t)r;
+    const size_t src = GATHER ? (size_t)(perm[r] / top) : (size_t)r;
     arow[j] = A + src * K + fq * 8;
   }
   float4v acc[4], accu[SWIGLU ? 4 : 1];
@@ -272,7 +295,8 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
     for (int i = 0; i < 4; ++i) {
       const int n = nb + 4 * fq + i;
       if (n < N) {
-        const float v = SWIGLU ? silu_f(acc[j][i]) * accu[j][i] : acc[j][i];
+        const float v = SWIGLU ? silu_f(acc[j][i]) * accu[j][i]
+                               : MODE == 2 ? relu2_f(acc[j][i]) : acc[j][i];
         out[(size_t)r * N + n] = f2bf(v);
       }
     }
@@ -291,10 +315,12 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma_kernel(
 #define GG_KC 64
 #define GG_NF 2
 
-template <int SWIGLU>
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wt, const int* __restrict__ plan, int P,
     int E, int top, int K, int N, bf16_t* __restrict__ out) {
+  constexpr int SWIGLU = MODE == 1;
+  constexpr bool GATHER = MODE != 0;
   __shared__ __attribute__((aligned(16))) bf16_t rows[GG_R2][GG_KC + 8];
   const int* offsets = plan;
   const int* perm = plan + E + 2;
@@ -329,7 +355,7 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
     srr[j] = i >> 3;
     scc[j] = (i & 7) * 8;
     const int r = min(r0 + srr[j], r1 - 1);
-    const size_t src = SWIGLU ? (size_t)(perm[r] / top) : (size_t)r;
+    const size_t src = GATHER ? (size_t)(perm[r] / top) : (size_t)r;
     srow[j] = A + src * K + scc[j];
   }
   float4v acc[GG_NF][8], accu[SWIGLU ? GG_NF : 1][SWIGLU ? 8 : 1];
@@ -407,7 +433,8 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
       for (int i = 0; i < 4; ++i) {
         const int n = nb + 16 * f + 4 * fq + i;
         if (n < N) {
-          const float v = SWIGLU ? silu_f(acc[f][j][i]) * accu[f][j][i] : acc[f][j][i];
+          const float v = SWIGLU ? silu_f(acc[f][j][i]) * accu[f][j][i]
+                                 : MODE == 2 ? relu2_f(acc[f][j][i]) : acc[f][j][i];
           out[(size_t)r * N + n] = f2bf(v);
         }
       }
@@ -454,13 +481,14 @@ extern "C" int loqa_silu_mul_any(const void* x, int dt, int T, int F, void* y, h
   return (int)hipGetLastError();
 }
 
-extern "C" int loqa_moe_route(const void* z, const void* corr, int E, int G, int keep, int top,
-                              void* idx, void* wt, int T, hipStream_t st) {
+extern "C" int loqa_moe_route(const void* z, const void* corr, const void* bias, int top_softmax,
+                              int E, int G, int keep, int top, void* idx, void* wt, int T,
+                              hipStream_t st) {
   if (T <= 0) return 0;
   if (E > MOE_MAX_E || E <= 0 || G <= 0 || E % G || top <= 0 || top > E)
     return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(64), 0, st, (const float*)z, (const float*)corr,
-                     E, G, keep, top, (int*)idx, (float*)wt);
+                     (const float*)bias, top_softmax, E, G, keep, top, (int*)idx, (float*)wt);
   return (int)hipGetLastError();
 }
 
@@ -471,36 +499,43 @@ extern "C" int loqa_moe_plan(const void* idx, int P, int E, void* plan, hipStrea
 }
 
 extern "C" int loqa_moe_grouped_gemm(const void* A, int dt, const void* W, const void* plan, int P,
-                                     int E, int top, int K, int N, int swiglu, void* out,
+                                     int E, int top, int K, int N, int mode, void* out,
                                      hipStream_t st) {
   if (P <= 0) return 0;
+  if (mode < 0 || mode > 2) return (int)hipErrorInvalidValue;
   const dim3 grid((P + GG_T - 1) / GG_T + E, (N + GG_T - 1) / GG_T);
+#define BY_MODE(KERNEL, GRID, TT)                                                               \
+  do {                                                                                          \
+    if (mode == 1)                                                                              \
+      hipLaunchKernelGGL(KERNEL(1), GRID, dim3(256), 0, st, (const TT*)A, (const TT*)W,         \
+                         (const int*)plan, P, E, top, K, N, (TT*)out);                          \
+    else if (mode == 2)                                                                         \
+      hipLaunchKernelGGL(KERNEL(2), GRID, dim3(256), 0, st, (const TT*)A, (const TT*)W,         \
+                         (const int*)plan, P, E, top, K, N, (TT*)out);                          \
+    else                                                                                        \
+      hipLaunchKernelGGL(KERNEL(0), GRID, dim3(256), 0, st, (const TT*)A, (const TT*)W,         \
+                         (const int*)plan, P, E, top, K, N, (TT*)out);                          \
+  } while (0)
+#define K_MFMA2(M) (moe_grouped_gemm_mfma2_kernel<M>)
+#define K_MFMA(M) (moe_grouped_gemm_mfma_kernel<M>)
+#define K_BF16(M) (moe_grouped_gemm_kernel<bf16_t, M>)
+#define K_F32(M) (moe_grouped_gemm_kernel<float, M>)
   if (dt == 0 && K % GG_KC == 0 && P >= 16 * (E > 0 ? E : 1) * 4 && P >= 1024) {
     // prompt-sized: on average at least 64 rows per expert
     const dim3 g2((P + GG_R2 - 1) / GG_R2 + E, (N + 64 * GG_NF - 1) / (64 * GG_NF));
-    if (swiglu)
-      hipLaunchKernelGGL(moe_grouped_gemm_mfma2_kernel<1>, g2, dim3(256), 0, st, (const bf16_t*)A,
-                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
-    else
-      hipLaunchKernelGGL(moe_grouped_gemm_mfma2_kernel<0>, g2, dim3(256), 0, st, (const bf16_t*)A,
-                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
-    return (int)hipGetLastError();
+    BY_MODE(K_MFMA2, g2, bf16_t);
+  } else if (dt == 0 && K >= 32 && K % 32 == 0) {
+    BY_MODE(K_MFMA, grid, bf16_t);
+  } else if (dt == 0) {
+    BY_MODE(K_BF16, grid, bf16_t);
+  } else {
+    BY_MODE(K_F32, grid, float);
   }
-  if (dt == 0 && K >= 32 && K % 32 == 0) {
-    if (swiglu)
-      hipLaunchKernelGGL(moe_grouped_gemm_mfma_kernel<1>, grid, dim3(256), 0, st, (const bf16_t*)A,
-                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
-    else
-      hipLaunchKernelGGL(moe_grouped_gemm_mfma_kernel<0>, grid, dim3(256), 0, st, (const bf16_t*)A,
-                         (const bf16_t*)W, (const int*)plan, P, E, top, K, N, (bf16_t*)out);
-    return (int)hipGetLastError();
-  }
-#define GO(TT, SW)                                                                              \
-  hipLaunchKernelGGL((moe_grouped_gemm_kernel<TT, SW>), grid, dim3(256), 0, st, (const TT*)A,   \
-                     (const TT*)W, (const int*)plan, P, E, top, K, N, (TT*)out)
-  if (dt == 0) { if (swiglu) GO(bf16_t, 1); else GO(bf16_t, 0); }
-  else { if (swiglu) GO(float, 1); else GO(float, 0); }
-#undef GO
+#undef K_MFMA2
+#undef K_MFMA
+#undef K_BF16
+#undef K_F32
+#undef BY_MODE
   return (int)hipGetLastError();
 }
 

@@ -220,10 +220,19 @@ _SEQMIX_SIGS = {
     "loqa_lightning_scan": [_vp, _l, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "loqa_gated_rmsnorm": [_vp, _vp, _vp, _i, _l, _f, _vp, _i, _i, _i, _vp],
     "loqa_silu_mul_any": [_vp, _i, _i, _i, _vp, _vp],
-    "loqa_moe_route": [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp],
+    "loqa_moe_route": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp],
     "loqa_moe_plan": [_vp, _i, _i, _vp, _vp],
     "loqa_moe_grouped_gemm": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp],
     "loqa_moe_combine": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
+    "loqa_token_shift": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp],
+    "loqa_seq_state_save": [_vp, _i, _vp, _i, _i, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _vp],
+    "loqa_conv_norm_rope_append": [_vp, _i, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp,
+                                   _f, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _vp, _i,
+                                   _vp],
+    "loqa_sigmoid_attention": [_vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i,
+                               _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp],
+    "loqa_scalar_rms_add": [_vp, _vp, _i, _f, _f, _vp, _i, _i, _vp],
+    "loqa_scalar_rms_norm": [_vp, _vp, _f, _f, _vp, _i, _i, _vp],
 }
 _seqmix = None
 
