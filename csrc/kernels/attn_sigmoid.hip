@@ -8,17 +8,20 @@
 // through the block table, so prompt portions, decode tokens and mixed batches
 // are one launch.
 //
-// Two forms:
+// Three forms:
 //  * sigmoid_attn_rows_kernel (any dtype, any head size): a wave per (token,
 //    head), four heads per workgroup. Lanes take one key each for the scores
-//    (f32 dot products, 16-byte loads of the key row), the weights of up to 64
-//    keys go through LDS, then lanes take output columns and add the weighted
-//    value rows in ascending key order. This is the decode form and the exact
-//    f32 form.
-//  * sigmoid_attn_mfma_kernel (bf16, D = 64 / 128): a workgroup per (16-row
-//    query tile of one sequence, key/value head); its waves share the staged K
-//    and (transposed) V tiles of 32 keys in LDS and take the query heads of the
-//    group in turn. S^T = K Q^T and O^T = V^T P^T run on
+//    (f32 dot products), the weights of up to 64 keys go through LDS, then
+//    lanes take output columns and add the weighted value rows in ascending
+//    key order. The form for head sizes the others do not take.
+//  * sigmoid_attn_keys_kernel (any dtype, D a power of two): the decode form
+//    and the exact f32 form; see there.
+//  * sigmoid_attn_mfma_kernel (bf16, D = 64 / 128): a workgroup per (64 query
+//    rows of one sequence, key/value head); each wave owns a 16-row tile and
+//    carries the group's query heads in registers, all waves share the staged
+//    K and (transposed) V tiles of 64 keys in LDS (the next tile's rows are in
+//    flight in registers), and a wave skips the steps that lie before its
+//    rows' chunk or after them. S^T = K Q^T and O^T = V^T P^T run on
 //    v_mfma_f32_16x16x32_bf16; the key order inside a 32-key step is permuted
 //    so that the score accumulators ARE the P^T operand (no shuffles). Scores,
 //    sigmoid and the output accumulators are f32.
@@ -55,7 +58,7 @@ __global__ __launch_bounds__(256) void sigmoid_attn_rows_kernel(SigAttnParams p)
   const float hb = p.bias[h];
   const T* kc = (const T*)p.kc;
   const T* vc = (const T*)p.vc;
-  constexpr int NV = 4;                          // output columns per lane (D <= 256)
+  constexpr int NV = 8;                          // output columns per lane (D <= 512)
   float acc[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) acc[i] = 0.f;
@@ -104,42 +107,167 @@ __global__ __launch_bounds__(256) void sigmoid_attn_rows_kernel(SigAttnParams p)
   }
 }
 
-// ------------------------------------------------------------ matrix cores
-#define SA_KT 32                                 // keys per step
-#define SA_VP 8                                  // padding (elements) of a transposed V row
 
-template <int D, int UPW>
-__global__ __launch_bounds__(256) void sigmoid_attn_mfma_kernel(SigAttnParams p, int tiles_per_seq,
+// ------------------------------------------------------------ few rows, many keys
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float* f) {
+    unpack8(*reinterpret_cast<const uint4*>(p), f);
+  }
+};
+template <> struct Vec8<float> {
+  static __device__ __forceinline__ void ld(const float* p, float* f) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  }
+};
+
+// The decode form (D a power of two, 8 .. 512): a workgroup per (token,
+// key/value head) serves up to RH query heads of the group, so every K and V row
+// is read once for all of them. The visible keys go in tiles of 64, dealt to
+// the workgroup's waves in turn. Scores: a lane takes one key and all RH heads (16-byte
+// loads of the key row against the queries in LDS). Values: the lanes regroup
+// as (key subgroup, 8 output columns), every lane adds its keys' value rows
+// weighted from LDS, and the partial sums meet through shuffles (key
+// subgroups), then LDS (waves), in a fixed order. Which wave, lane and step a
+// key lands on depends only on its offset from the chunk's first key.
+template <typename T, int RH, int DC>
+__global__ __launch_bounds__(512) void sigmoid_attn_keys_kernel(SigAttnParams p, int heads_per_wg) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, NW = blockDim.x >> 6;
+  const int t = blockIdx.x, g = blockIdx.y;
+  if (t >= p.cu_q[p.B]) return;
+  int b = 0;
+  while (b + 1 < p.B && t >= p.cu_q[b + 1]) ++b;
+  const int D = DC ? DC : p.D;                   // head sizes 64 and 128 unroll fully
+  const int GD = p.G * D, HD = p.H * D, rep = p.H / p.G;
+  const int h_first = g * rep + blockIdx.z * heads_per_wg;
+  const int nh = min(heads_per_wg, g * rep + rep - h_first);
+  float* qs = lds;                               // [RH][D]
+  float* red = qs + RH * D;                      // [NW][RH][D]
+  float* wts = red + NW * RH * D + wave * (RH + 1) * 64;     // per wave [RH][64] weights
+  int* rowi = reinterpret_cast<int*>(wts + RH * 64);         // per wave [64] cache rows
+  const T* q = (const T*)p.q + (size_t)t * HD + (size_t)h_first * D;
+  for (int i = threadIdx.x; i < nh * D; i += blockDim.x) qs[i] = Act<T>::ld(q + i);
+  __syncthreads();
+  const int pq = p.pos[t];
+  const int lo = chunk_start(pq, p.chunk), hi = min(pq, p.ctx[b] - 1);
+  const int ntiles = hi >= lo ? (hi - lo) / 64 + 1 : 0;
+  const int* bt = p.bt + (size_t)b * p.max_blocks;
+  const T* kc = (const T*)p.kc;
+  const T* vc = (const T*)p.vc;
+  const int CG = D / 8, KS = 64 / CG;            // column groups, key subgroups
+  const int cgi = lane % CG, ksi = lane / CG;
+  float hb[RH];
+#pragma unroll
+  for (int r = 0; r < RH; ++r) hb[r] = p.bias[min(h_first + r, p.H - 1)];
+  float acc[RH][8];
+#pragma unroll
+  for (int r = 0; r < RH; ++r)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
+  for (int tile = wave; tile < ntiles; tile += NW) {
+    const int k0 = lo + 64 * tile, j = k0 + lane;
+    float sc[RH];
+#pragma unroll
+    for (int r = 0; r < RH; ++r) sc[r] = 0.f;
+    int row = 0;
+    if (j <= hi) {
+      row = (int)min(max((long)bt[j / p.blk] * p.blk + j % p.blk, 0L), p.cache_rows - 1);
+      const T* kr = kc + (size_t)row * GD + (size_t)g * D;
+#pragma unroll(DC ? DC / 8 : 4)
+      for (int e = 0; e < D; e += 8) {
+        float f[8];
+        Vec8<T>::ld(kr + e, f);
+#pragma unroll
+        for (int r = 0; r < RH; ++r)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sc[r] += qs[r * D + e + i] * f[i];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RH; ++r)
+      wts[r * 64 + lane] = j <= hi && r < nh ? sigmoid_for<T>(sc[r] * p.scale + hb[r]) : 0.f;
+    rowi[lane] = row;                            // lanes past the last key: weight 0 on row 0
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll(DC ? DC / 8 : 4)
+    for (int kk = ksi; kk < 64; kk += KS) {
+      float f[8];
+      Vec8<T>::ld(vc + (size_t)rowi[kk] * GD + (size_t)g * D + cgi * 8, f);
+#pragma unroll
+      for (int r = 0; r < RH; ++r) {
+        const float w = wts[r * 64 + kk];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[r][i] += w * f[i];
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  for (int off = CG; off < 64; off <<= 1)
+#pragma unroll
+    for (int r = 0; r < RH; ++r)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[r][i] += __shfl_xor(acc[r][i], off, 64);
+  if (ksi == 0)
+#pragma unroll
+    for (int r = 0; r < RH; ++r)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) red[(wave * RH + r) * D + cgi * 8 + i] = acc[r][i];
+  __syncthreads();
+  for (int i = threadIdx.x; i < nh * D; i += blockDim.x) {
+    const int r = i / D, e = i % D, h = h_first + r;
+    float v = 0.f;
+    for (int w = 0; w < NW; ++w) v += red[(w * RH + r) * D + e];       // waves in order
+    float gt = 1.f;
+    if (p.gate) gt = sigmoid_f(Act<T>::ld((const T*)p.gate + (size_t)t * p.gate_ld + h));
+    Act<T>::st((T*)p.o + (size_t)t * HD + (size_t)h * D + e, v * gt);
+  }
+}
+
+// ------------------------------------------------------------ matrix cores
+#define SA_KT 64                                 // keys staged per step (two 32-key MFMA sub-steps)
+#define SA_VP 2                                  // a transposed V row is 33 dwords: column writes spread over banks
+#define SA_ROWS 64                               // query rows per workgroup: one 16-row tile per wave
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// NH = query heads a wave carries (all of them against its own 16-row tile).
+template <int D, int NH>
+__global__ __launch_bounds__(256) void sigmoid_attn_mfma_kernel(SigAttnParams p, int blocks_per_seq,
                                                                 int heads_per_wg) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[SA_KT][D + 8];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[D][SA_KT + SA_VP];
-  const int b = blockIdx.x / tiles_per_seq, tile = blockIdx.x % tiles_per_seq;
+  constexpr int NCH = SA_KT * (D / 8) / 256;     // 16-byte chunks a thread stages per tile
+  const int b = blockIdx.x / blocks_per_seq, blk_i = blockIdx.x % blocks_per_seq;
   const int q0 = p.cu_q[b], n = p.cu_q[b + 1] - q0;
-  if (tile * 16 >= n) return;
-  const int t0 = q0 + tile * 16, nv = min(16, n - tile * 16);
+  if (blk_i * SA_ROWS >= n) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int r0 = blk_i * SA_ROWS;                               // first row of the block in the feed
+  const int nb = min(SA_ROWS, n - r0);                          // rows of the block
+  const int nv = max(0, min(16, nb - 16 * wave));               // rows of this wave's tile
   const int g = blockIdx.y, rep = p.H / p.G;
   const int h_first = g * rep + blockIdx.z * heads_per_wg;
   const int h_end = min(g * rep + rep, h_first + heads_per_wg);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int fr = lane & 15, fq = lane >> 4;
   const int GD = p.G * D, HD = p.H * D;
   const bf16_t* kc = (const bf16_t*)p.kc;
   const bf16_t* vc = (const bf16_t*)p.vc;
   const int* bt = p.bt + (size_t)b * p.max_blocks;
-  const int ctx = p.ctx[b];
-  const int p0 = p.pos[t0];                      // rows of a feed hold consecutive positions
-  const int pq = p0 + min(fr, nv - 1);           // this lane's query (clamped rows repeat the last)
+  const int p0 = p.pos[q0 + r0];                 // rows of a feed hold consecutive positions
+  const int kbeg = chunk_start(p0, p.chunk), kend = min(p0 + nb - 1, p.ctx[b] - 1);
+  // this wave's tile: positions pw0 .. pw1; this lane's query (clamped rows repeat the last)
+  const int pw0 = p0 + 16 * wave, pw1 = pw0 + max(nv, 1) - 1;
+  const int wlo = chunk_start(pw0, p.chunk);
+  const int pq = pw0 + min(fr, max(nv, 1) - 1);
   const int lo_q = chunk_start(pq, p.chunk);
-  const int kbeg = chunk_start(p0, p.chunk), kend = min(p0 + nv - 1, ctx - 1);
 
-  // this wave's heads: h_first + wave, + 4, ...; their query fragments and accumulators
-  bf16x8 qf[UPW][D / 32];
-  float4v oacc[UPW][D / 16];
-  float hb[UPW];
-  const bf16_t* qrow = (const bf16_t*)p.q + (size_t)(t0 + min(fr, nv - 1)) * HD + fq * 8;
+  bf16x8 qf[NH][D / 32];
+  float4v oacc[NH][D / 16];
+  float hb[NH];
+  const int trow = q0 + r0 + min(16 * wave + min(fr, max(nv, 1) - 1), nb - 1);
+  const bf16_t* qrow = (const bf16_t*)p.q + (size_t)trow * HD + fq * 8;
 #pragma unroll
-  for (int u = 0; u < UPW; ++u) {
-    const int h = min(h_first + wave + 4 * u, p.H - 1);
+  for (int u = 0; u < NH; ++u) {
+    const int h = min(h_first + u, p.H - 1);
     hb[u] = p.bias[h];
 #pragma unroll
     for (int ks = 0; ks < D / 32; ++ks)
@@ -148,69 +276,97 @@ __global__ __launch_bounds__(256) void sigmoid_attn_mfma_kernel(SigAttnParams p,
     for (int et = 0; et < D / 16; ++et) oacc[u][et] = float4v{0.f, 0.f, 0.f, 0.f};
   }
 
+  // staging: thread -> NCH chunks (key, 8 entries) of K and of V; the next
+  // tile's rows are requested before this tile's MFMAs and land in LDS after them
+  u32x4 kreg[NCH], vreg[NCH];           // (plain vectors: these stay in registers)
+  // (rows past the last key repeat it: their weights are zero; no branch, so
+  // the block-table lookups and then all row loads are in flight together)
+#define SA_FETCH(K0)                                                                            \
+  {                                                                                             \
+    long row_[NCH];                                                                             \
+    _Pragma("unroll") for (int c = 0; c < NCH; ++c) {                                           \
+      const int j_ = min((K0) + (int)(threadIdx.x + 256 * c) / (D / 8), kend);                  \
+      row_[c] = min(max((long)bt[j_ / p.blk] * p.blk + j_ % p.blk, 0L), p.cache_rows - 1);      \
+    }                                                                                           \
+    _Pragma("unroll") for (int c = 0; c < NCH; ++c) {                                           \
+      const int ch_ = ((threadIdx.x + 256 * c) % (D / 8)) * 8;                                  \
+      kreg[c] = *reinterpret_cast<const u32x4*>(kc + (size_t)row_[c] * GD + (size_t)g * D + ch_); \
+      vreg[c] = *reinterpret_cast<const u32x4*>(vc + (size_t)row_[c] * GD + (size_t)g * D + ch_); \
+    }                                                                                           \
+  }
+  SA_FETCH(kbeg)
   for (int k0 = kbeg; k0 <= kend; k0 += SA_KT) {
     __syncthreads();                             // the previous step's tiles are consumed
-    // stage 32 key rows: K as it is, V transposed; 16-byte chunks of 8 entries
-    for (int i = threadIdx.x; i < SA_KT * (D / 8); i += 256) {
-      const int key = i / (D / 8), ch = (i % (D / 8)) * 8;
-      const int j = k0 + key;
-      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (j <= kend) {
-        const long row = min(max((long)bt[j / p.blk] * p.blk + j % p.blk, 0L), p.cache_rows - 1);
-        kv = *reinterpret_cast<const uint4*>(kc + (size_t)row * GD + (size_t)g * D + ch);
-        vv = *reinterpret_cast<const uint4*>(vc + (size_t)row * GD + (size_t)g * D + ch);
-      }
-      *reinterpret_cast<uint4*>(&Ks[key][ch]) = kv;
-      const bf16_t* ve = reinterpret_cast<const bf16_t*>(&vv);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) Vt[ch + e][key] = ve[e];
+    for (int c = 0; c < NCH; ++c) {
+      const int i = threadIdx.x + 256 * c;
+      const int key = i / (D / 8), ch = (i % (D / 8)) * 8;
+      *reinterpret_cast<u32x4*>(&Ks[key][ch]) = kreg[c];
+#define SA_PUT(E, W)                                    \
+  Vt[ch + 2 * (E)][key] = (bf16_t)((W) & 0xffffu);      \
+  Vt[ch + 2 * (E) + 1][key] = (bf16_t)((W) >> 16);
+      SA_PUT(0, vreg[c].x) SA_PUT(1, vreg[c].y) SA_PUT(2, vreg[c].z) SA_PUT(3, vreg[c].w)
+#undef SA_PUT
     }
     __syncthreads();
+    if (k0 + SA_KT <= kend) { SA_FETCH(k0 + SA_KT) }
+    if (nv == 0) continue;
 #pragma unroll
-    for (int u = 0; u < UPW; ++u) {
-      if (h_first + wave + 4 * u >= h_end) continue;        // wave-uniform
-      // S^T tiles: keys k0 + 16 kt + 4 fq + i against query fr
-      float4v s[2];
+    for (int sub = 0; sub < SA_KT / 32; ++sub) {
+      const int ks0 = k0 + 32 * sub;             // first key of this 32-key sub-step
+      // nothing of it is visible to the wave's rows: after them or before their chunk
+      if (ks0 > pw1 || ks0 + 32 <= wlo) continue;
+      // S^T tiles: keys ks0 + 16 kt + 4 fq + i against query fr; a K fragment
+      // read from LDS serves every head the wave carries
+      float4v sc[NH][2];
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        s[kt] = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < D / 32; ++ks) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(&Ks[16 * kt + fr][32 * ks + fq * 8]);
-          s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[u][ks], s[kt], 0, 0, 0);
-        }
-      }
-      // weights in f32, then the P^T operand: slot kk < 4 is key 4 fq + kk,
-      // slot kk >= 4 is key 16 + 4 fq + kk - 4 (the V^T operand uses the same order)
-      float w[2][4];
+      for (int u = 0; u < NH; ++u) sc[u][0] = sc[u][1] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int j = k0 + 16 * kt + 4 * fq + i;
-          const bool seen = j <= pq && j >= lo_q;
-          w[kt][i] = seen ? sigmoid_f(s[kt][i] * p.scale + hb[u]) : 0.f;
+        for (int ks = 0; ks < D / 32; ++ks) {
+          const bf16x8 a = *reinterpret_cast<const bf16x8*>(
+              &Ks[32 * sub + 16 * kt + fr][32 * ks + fq * 8]);
+#pragma unroll
+          for (int u = 0; u < NH; ++u)
+            sc[u][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[u][ks], sc[u][kt], 0, 0, 0);
         }
-      uint4 pu;
-      pu.x = pack_bf16x2(w[0][0], w[0][1]); pu.y = pack_bf16x2(w[0][2], w[0][3]);
-      pu.z = pack_bf16x2(w[1][0], w[1][1]); pu.w = pack_bf16x2(w[1][2], w[1][3]);
-      const bf16x8 pw = *reinterpret_cast<const bf16x8*>(&pu);
+      // weights in f32, then the P^T operands: slot kk < 4 is key 4 fq + kk,
+      // slot kk >= 4 is key 16 + 4 fq + kk - 4 (the V^T operand uses the same order)
+      bf16x8 pw[NH];
+#pragma unroll
+      for (int u = 0; u < NH; ++u) {
+        float w[2][4];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int j = ks0 + 16 * kt + 4 * fq + i;
+            const bool seen = j <= pq && j >= lo_q;
+            w[kt][i] = seen ? sigmoid_fast(sc[u][kt][i] * p.scale + hb[u]) : 0.f;
+          }
+        const u32x4 pu = {pack_bf16x2(w[0][0], w[0][1]), pack_bf16x2(w[0][2], w[0][3]),
+                          pack_bf16x2(w[1][0], w[1][1]), pack_bf16x2(w[1][2], w[1][3])};
+        pw[u] = __builtin_bit_cast(bf16x8, pu);
+      }
 #pragma unroll
       for (int et = 0; et < D / 16; ++et) {
-        const uint2 v0 = *reinterpret_cast<const uint2*>(&Vt[16 * et + fr][4 * fq]);
-        const uint2 v1 = *reinterpret_cast<const uint2*>(&Vt[16 * et + fr][16 + 4 * fq]);
-        uint4 va = make_uint4(v0.x, v0.y, v1.x, v1.y);
-        oacc[u][et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            *reinterpret_cast<const bf16x8*>(&va), pw, oacc[u][et], 0, 0, 0);
+        const uint32_t* vr = reinterpret_cast<const uint32_t*>(&Vt[16 * et + fr][32 * sub]);
+        const u32x4 va = {vr[2 * fq], vr[2 * fq + 1], vr[8 + 2 * fq], vr[9 + 2 * fq]};
+#pragma unroll
+        for (int u = 0; u < NH; ++u)
+          oacc[u][et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, va), pw[u], oacc[u][et], 0, 0, 0);
       }
     }
   }
+#undef SA_FETCH
   // oacc[u][et][i]: output column 16 et + 4 fq + i of query row fr
   if (fr >= nv) return;
-  const int t = t0 + fr;
+  const int t = q0 + r0 + 16 * wave + fr;
 #pragma unroll
-  for (int u = 0; u < UPW; ++u) {
-    const int h = h_first + wave + 4 * u;
+  for (int u = 0; u < NH; ++u) {
+    const int h = h_first + u;
     if (h >= h_end) continue;
     float gt = 1.f;
     if (p.gate) gt = sigmoid_f(bf2f(((const bf16_t*)p.gate)[(size_t)t * p.gate_ld + h]));
@@ -231,7 +387,7 @@ extern "C" int loqa_sigmoid_attention(
     const void* gate, int gate_ld, float scale, int chunk, int B, int T, int H, int G, int D,
     int max_q, int mfma, void* o, hipStream_t st) {
   if (T <= 0) return 0;
-  if (B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > 256 || blk <= 0 || nblocks <= 0 ||
+  if (B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > 512 || blk <= 0 || nblocks <= 0 ||
       chunk < 0)
     return (int)hipErrorInvalidValue;
   SigAttnParams p;
@@ -242,15 +398,53 @@ extern "C" int loqa_sigmoid_attention(
   p.D = D; p.o = o;
   if (mfma && dt == 0 && (D == 64 || D == 128) && max_q > 0) {
     const int rep = H / G;
-    const int zs = (rep + 15) / 16;                        // at most 16 heads per workgroup
+    const int hmax = D == 64 ? 8 : 4;                      // heads a wave can carry in registers
+    const int blocks = (max_q + SA_ROWS - 1) / SA_ROWS;
+    int zs = (rep + hmax - 1) / hmax;
+    int hpw = (rep + zs - 1) / zs;
+    // a short batch fills the chip through more, narrower workgroups: the query
+    // heads of a group spread over workgroups (K / V tiles come from L2 again)
+    while (hpw > 1 && (long)B * blocks * G * zs < 256) {
+      hpw = (hpw + 1) / 2;
+      zs = (rep + hpw - 1) / hpw;
+    }
+    const dim3 grid(B * blocks, G, zs);
+#define GO(DD, NN)                                                                              \
+  hipLaunchKernelGGL((sigmoid_attn_mfma_kernel<DD, NN>), grid, dim3(256), 0, st, p, blocks, hpw)
+    if (D == 64) {
+      if (hpw <= 1) GO(64, 1); else if (hpw == 2) GO(64, 2); else if (hpw <= 4) GO(64, 4);
+      else GO(64, 8);
+    } else {
+      if (hpw <= 1) GO(128, 1); else if (hpw == 2) GO(128, 2); else GO(128, 4);
+    }
+#undef GO
+    return (int)hipGetLastError();
+  }
+  if (D >= 8 && (D & (D - 1)) == 0) {
+    const int rep = H / G;
+    const int nw = D <= 128 ? 8 : 4;                       // waves: key tiles in flight
+    int rh = rep < 8 ? rep : 8;
+    if (rh * D > 1024 && nw == 8) rh = 1024 / D;           // LDS: (1 + nw) RH D floats
+    if (rh * D > 2048) rh = 2048 / D;
+    const int zs = (rep + rh - 1) / rh;
     const int hpw = (rep + zs - 1) / zs;
-    const int upw = (hpw + 3) / 4;
-    const int tiles = (max_q + 15) / 16;
-    const dim3 grid(B * tiles, G, zs);
-#define GO(DD, UU)                                                                              \
-  hipLaunchKernelGGL((sigmoid_attn_mfma_kernel<DD, UU>), grid, dim3(256), 0, st, p, tiles, hpw)
-    if (D == 64) { if (upw <= 1) GO(64, 1); else if (upw == 2) GO(64, 2); else GO(64, 4); }
-    else { if (upw <= 1) GO(128, 1); else if (upw == 2) GO(128, 2); else GO(128, 4); }
+    const int RH = hpw <= 1 ? 1 : hpw == 2 ? 2 : hpw <= 4 ? 4 : 8;
+    const dim3 grid(T, G, zs);
+    const size_t lds = ((size_t)(1 + nw) * RH * D + nw * (RH + 1) * 64) * sizeof(float);
+#define GO(TT, RR, DD)                                                                          \
+  hipLaunchKernelGGL((sigmoid_attn_keys_kernel<TT, RR, DD>), grid, dim3(64 * nw), lds, st, p, hpw)
+#define BY_D(TT, RR)                                                                            \
+  do {                                                                                          \
+    if (D == 64) GO(TT, RR, 64); else if (D == 128) GO(TT, RR, 128); else GO(TT, RR, 0);        \
+  } while (0)
+#define BY_RH(TT)                                                                               \
+  do {                                                                                          \
+    if (RH == 1) BY_D(TT, 1); else if (RH == 2) BY_D(TT, 2); else if (RH == 4) BY_D(TT, 4);     \
+    else BY_D(TT, 8);                                                                           \
+  } while (0)
+    if (dt == 0) BY_RH(bf16_t); else BY_RH(float);
+#undef BY_RH
+#undef BY_D
 #undef GO
     return (int)hipGetLastError();
   }

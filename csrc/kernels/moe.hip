@@ -366,9 +366,10 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
       acc[f][j] = float4v{0.f, 0.f, 0.f, 0.f};
       if (SWIGLU) accu[f][j] = float4v{0.f, 0.f, 0.f, 0.f};
     }
-  uint4 pre[4];
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 pre[4];                                  // (a plain vector type: stays in registers)
 #pragma unroll
-  for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j]);
+  for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const u32x4*>(srow[j]);
   // this chunk's weight fragments (2 k-steps); the next chunk's are requested
   // before this chunk's MFMAs, so the weight stream's latency stays hidden
   bf16x8 wa[2][GG_NF], wb[SWIGLU ? 2 : 1][GG_NF];
@@ -382,13 +383,13 @@ __global__ __launch_bounds__(256) void moe_grouped_gemm_mfma2_kernel(
   for (int k0 = 0; k0 < K; k0 += GG_KC) {
     __syncthreads();                                     // the previous chunk is consumed
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(&rows[srr[j]][scc[j]]) = pre[j];
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(&rows[srr[j]][scc[j]]) = pre[j];
     __syncthreads();
     const bool more = k0 + GG_KC < K;
     bf16x8 na[2][GG_NF], nb2[SWIGLU ? 2 : 1][GG_NF];
     if (more) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const uint4*>(srow[j] + k0 + GG_KC);
+      for (int j = 0; j < 4; ++j) pre[j] = *reinterpret_cast<const u32x4*>(srow[j] + k0 + GG_KC);
 #pragma unroll
       for (int q = 0; q < 2; ++q)
 #pragma unroll

@@ -11,9 +11,12 @@
 // so a step never sees half-updated state.
 //
 // conv_norm_rope_append_kernel (one workgroup per token) is everything between
-// the q | k projection GEMM and attention: convolution in f32, v = convolved k,
-// RMS norm over the whole q and the whole k projection, rotate-half rotary
-// positions on the first `dims` entries of every head, k and v into their pages.
+// the q | k projection GEMM and attention: convolution in f32 (weights stored
+// tap-major, [taps][C]), v = convolved k, RMS norm over the whole q and the
+// whole k projection, rotate-half rotary positions on the first `dims` entries
+// of every head, k and v into their pages. The v8 form gives a thread 8
+// neighbouring channels (16-byte loads and stores, all taps' loads in flight at
+// once); the scalar form takes any sizes.
 #include "seqmix.h"
 
 __device__ __forceinline__ int seq_of_row(const int* __restrict__ cu_q, int B, int t) {
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(256) void conv_norm_rope_append_kernel(
       if (p - s < 0) continue;                    // before the sequence's start
       const float uv = i - s >= 0 ? Act<TU>::ld(u + (size_t)(t - s) * ldu + c)
                                   : ts[(size_t)(keep + i - s) * C + c];
-      acc += cw[(size_t)c * taps + j] * uv;
+      acc += cw[(size_t)j * C + c] * uv;
     }
     y[c] = acc;
     if (c < Cq) sq += acc * acc; else sk += acc * acc;
@@ -122,6 +125,111 @@ __global__ __launch_bounds__(256) void conv_norm_rope_append_kernel(
     else if (store) {
       Act<TO>::st(kc + (size_t)slot * Ck + cc, v);
       Act<TO>::st(vc + (size_t)slot * Ck + cc, y[c]);
+    }
+  }
+}
+
+
+template <typename T> struct Row8;
+template <> struct Row8<bf16_t> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float* f) {
+    unpack8(*reinterpret_cast<const uint4*>(p), f);
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, const float* f) {
+    *reinterpret_cast<uint4*>(p) = pack8(f);
+  }
+};
+template <> struct Row8<float> {
+  static __device__ __forceinline__ void ld(const float* p, float* f) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  }
+  static __device__ __forceinline__ void st(float* p, const float* f) {
+    *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
+  }
+};
+
+// D, ldu and so C are multiples of 8: a thread's 8 channels lie in one head.
+template <typename TU, typename TO>
+__global__ __launch_bounds__(1024) void conv_norm_rope_append_v8_kernel(
+    const TU* __restrict__ u, int ldu, const float* __restrict__ cw, int taps,
+    const float* __restrict__ tail, int nslots, const int* __restrict__ sslots,
+    const int* __restrict__ cu_q, const int* __restrict__ pos, int B,
+    const float* __restrict__ qn, const float* __restrict__ kn, float eps,
+    const float* __restrict__ cs, int max_pos, int dims, int H, int G, int D,
+    TO* __restrict__ kc, TO* __restrict__ vc, long cache_rows, const int* __restrict__ kvslots,
+    TO* __restrict__ q) {
+  extern __shared__ float y[];
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  if (t >= cu_q[B]) return;
+  const int b = seq_of_row(cu_q, B, t);
+  const int i = t - cu_q[b], p = pos[t], keep = taps - 1;
+  const int Cq = H * D, Ck = G * D, C = Cq + Ck;
+  const float* ts = tail + (size_t)min(max(sslots[b], 0), nslots - 1) * keep * C;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x * 8; c < C; c += blockDim.x * 8) {
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    if (i >= keep) {                             // every tap lies inside the feed: no branch
+#pragma unroll 4
+      for (int j = 0; j < taps; ++j) {
+        float uv[8], w[8];
+        Row8<TU>::ld(u + (size_t)(t - keep + j) * ldu + c, uv);
+        Row8<float>::ld(cw + (size_t)j * C + c, w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += w[e] * uv[e];
+      }
+    } else {
+      for (int j = max(0, keep - p); j < taps; ++j) {     // taps before position 0 read zeros
+        const int s = keep - j;
+        float uv[8], w[8];
+        if (i - s >= 0) Row8<TU>::ld(u + (size_t)(t - s) * ldu + c, uv);
+        else Row8<float>::ld(ts + (size_t)(keep + i - s) * C + c, uv);
+        Row8<float>::ld(cw + (size_t)j * C + c, w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += w[e] * uv[e];
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { y[c + e] = acc[e]; ss += acc[e] * acc[e]; }
+    if (c < Cq) sq += ss; else sk += ss;
+  }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);
+  const float rq = rsqrtf(sq / (float)Cq + eps), rk = rsqrtf(sk / (float)Ck + eps);
+  const int half = dims / 2;
+  const float* csp = cs + (size_t)min(max(p, 0), max_pos - 1) * dims;
+  const long slot = kvslots[t];
+  const bool store = slot >= 0 && slot < cache_rows;
+  for (int c = threadIdx.x * 8; c < C; c += blockDim.x * 8) {
+    const bool isq = c < Cq;
+    const int cc = isq ? c : c - Cq, e0 = cc % D;
+    const float r = isq ? rq : rk;
+    const float* nw = isq ? qn : kn;
+    float w[8], v[8], raw[8];
+    Row8<float>::ld(nw + cc, w);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { raw[e] = y[c + e]; v[e] = raw[e] * r * w[e]; }
+    if (e0 < dims) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = e0 + e;
+        if (d >= dims) continue;
+        const int f = d < half ? d : d - half;
+        const int off = d < half ? half : -half;
+        const float o = y[c + e + off] * r * nw[cc + e + off];
+        const float co = csp[2 * f], si = csp[2 * f + 1];
+        v[e] = d < half ? v[e] * co - o * si : v[e] * co + o * si;
+      }
+    }
+    if (isq) Row8<TO>::st(q + (size_t)t * Cq + c, v);
+    else if (store) {
+      Row8<TO>::st(kc + (size_t)slot * Ck + cc, v);
+      Row8<TO>::st(vc + (size_t)slot * Ck + cc, raw);
     }
   }
 }
@@ -170,15 +278,30 @@ extern "C" int loqa_conv_norm_rope_append(
       max_pos <= 0)
     return (int)hipErrorInvalidValue;
   const long rows = (long)blk * nblocks;
+  const bool v8 = D % 8 == 0 && ldu % 8 == 0;
+  int thr = 256;
+  if (v8) {
+    thr = (int)((C / 8 + 63) / 64) * 64;
+    if (thr > 1024) thr = 1024;
+  }
+#define ARGS(TU, TO)                                                                            \
+  (const TU*)u, ldu, (const float*)cw, taps, (const float*)tail, nslots, (const int*)sslots,    \
+      (const int*)cu_q, (const int*)pos, B, (const float*)qn, (const float*)kn, eps,            \
+      (const float*)cs, max_pos, dims, H, G, D, (TO*)kc, (TO*)vc, rows, (const int*)kvslots,    \
+      (TO*)q
 #define GO(TU, TO)                                                                              \
-  hipLaunchKernelGGL((conv_norm_rope_append_kernel<TU, TO>), dim3(T), dim3(256), C * 4, st,     \
-                     (const TU*)u, ldu, (const float*)cw, taps, (const float*)tail, nslots,     \
-                     (const int*)sslots, (const int*)cu_q, (const int*)pos, B, (const float*)qn, \
-                     (const float*)kn, eps, (const float*)cs, max_pos, dims, H, G, D, (TO*)kc,  \
-                     (TO*)vc, rows, (const int*)kvslots, (TO*)q)
+  do {                                                                                          \
+    if (v8)                                                                                     \
+      hipLaunchKernelGGL((conv_norm_rope_append_v8_kernel<TU, TO>), dim3(T), dim3(thr), C * 4,  \
+                         st, ARGS(TU, TO));                                                     \
+    else                                                                                        \
+      hipLaunchKernelGGL((conv_norm_rope_append_kernel<TU, TO>), dim3(T), dim3(256), C * 4, st, \
+                         ARGS(TU, TO));                                                         \
+  } while (0)
   if (u_dt == 0 && o_dt == 0) GO(bf16_t, bf16_t);
   else if (u_dt == 1 && o_dt == 1) GO(float, float);
   else return (int)hipErrorInvalidValue;
 #undef GO
+#undef ARGS
   return (int)hipGetLastError();
 }

@@ -25,5 +25,13 @@ template <> struct Act<float> {
 __device__ __forceinline__ float tanh_f(float z) { return 1.f - 2.f / (1.f + expf(2.f * z)); }
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+// The same through the hardware's exp2 and reciprocal (about 1 ulp each, a few
+// 1e-6 relative for |z| up to 50): for results that are rounded to bfloat16.
+__device__ __forceinline__ float sigmoid_fast(float z) {
+  return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896f * z));
+}
+template <typename T> __device__ __forceinline__ float sigmoid_for(float z) {
+  return sizeof(T) == 2 ? sigmoid_fast(z) : sigmoid_f(z);
+}
 
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

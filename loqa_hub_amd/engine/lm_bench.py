@@ -3,13 +3,14 @@ engine's step function, at layer sizes that resemble real models (random
 weights, synthetic tokens): ``python bench.py --lm-bench``.
 
 For each size a Pipizen stack (latent attention / lightning mixers, dense and
-mixture-of-experts feed-forwards) runs beside a Llama stack of the same width,
-depth, head count and feed-forward width - the framework's closest existing
-decoder. Measured per family:
+mixture-of-experts feed-forwards) and a Sodonex stack (chunked sigmoid
+attention with token shift and short convolutions, squared-relu experts) run
+beside a Llama stack of the same width, depth, head count and feed-forward
+width - the framework's plain decoder. Measured per family:
 
 * prefill: one prompt of ``P`` tokens through ``LLMEngine.step_logits``;
 * decode: ``B`` sequences at context ``P`` advancing one token per step
-  (Llama: the fused decode step the scheduler replays; Pipizen: its step
+  (Llama: the fused decode step the scheduler replays; the others: their step
   function on a [B]-row batch).
 
 One JSON line per (size, family); nothing here touches the default workload.
@@ -22,8 +23,9 @@ import time
 import numpy as np
 import torch
 
-from ..models.configs import (FeedForwardConfig, HybridLayerConfig, LatentAttnConfig, LightningConfig,
-                              LlamaConfig, PipizenConfig, RotaryConfig)
+from ..models.configs import (ChunkAttnConfig, FeedForwardConfig, HybridLayerConfig,
+                              LatentAttnConfig, LightningConfig, LlamaConfig, PipizenConfig,
+                              RotaryConfig, SodonexConfig)
 
 SIZES = {
     # name: (width, layers, heads, head_dim, rot_dim, kv_rank, ff, experts, expert_ff, top)
@@ -49,6 +51,17 @@ def pipizen_stack(name: str, vocab: int = 32000) -> PipizenConfig:
             FeedForwardConfig("moe", eff, E, 0, top, 4, 2, eff)
         layers.append(HybridLayerConfig(kind, mixer, mlp))
     return PipizenConfig(f"pipizen-{name}", vocab, d, 1e-6, tuple(layers))
+
+
+def sodonex_stack(name: str, vocab: int = 32000, chunk: int = 768) -> SodonexConfig:
+    """Every layer: grouped chunked sigmoid attention (4 query heads per
+    key/value head, 4 convolution taps) and the same experts as the Pipizen
+    stack's mixture layers (squared relu, no shared expert)."""
+    d, n, H, D, Dr, _, _, E, eff, top = SIZES[name]
+    mixer = ChunkAttnConfig(H, max(1, H // 4), D, D, 4, chunk, D ** -0.5, RotaryConfig(Dr, 10000.0))
+    mlp = FeedForwardConfig("moe", eff, E, 0, top, act="relu2", router="softmax_top")
+    return SodonexConfig(f"sodonex-{name}", vocab, d, 1e-6, 0.5, 1.0,
+                         tuple(HybridLayerConfig("attention", mixer, mlp) for _ in range(n)))
 
 
 def llama_stack(name: str, vocab: int = 32000) -> LlamaConfig:
@@ -118,7 +131,9 @@ def run(args) -> int:
         else torch.device("cpu")
     sizes = [s for s in args.lm_sizes.split(",") if s]
     for name in sizes:
-        for cfg in (pipizen_stack(name), llama_stack(name)):
+        fams = {"pipizen": pipizen_stack, "sodonex": sodonex_stack, "llama": llama_stack}
+        for fam in [f for f in args.lm_families.split(",") if f]:
+            cfg = fams[fam](name)
             if dev.type == "cpu":      # plumbing run: tiny stacks
                 prompt, batch, steps = 48, 2, 2
             else:

@@ -72,13 +72,18 @@ class SodonexWeights:
             wq, wk, wg = W(p + "mix.q"), W(p + "mix.k"), W(p + "mix.g")
             if wq.shape != (H * D, d) or wk.shape != (G * D, d) or wg.shape != (H, d):
                 raise ValueError(f"layer {i}: projection shapes do not match the config")
-            # q | k | gate rows as one GEMM (the gate has no bias)
-            L["wqkg"] = torch.cat([wq, wk, wg]).contiguous()
+            # q | k | gate rows as one GEMM (the gate has no bias); zero rows pad
+            # the output to a multiple of 8 columns so that its rows stay
+            # 16-byte aligned for the kernels that read them
+            pad = -H % 8
+            L["wqkg"] = torch.cat([wq, wk, wg, torch.zeros(pad, d, dtype=dtype, device=dev)]
+                                  ).contiguous()
             L["bqkg"] = torch.cat([W(p + "mix.q.b"), W(p + "mix.k.b"),
-                                   torch.zeros(H, dtype=dtype, device=dev)]).contiguous()
-            L["conv"] = torch.cat([F(p + "mix.q.conv"), F(p + "mix.k.conv")]).contiguous()
-            if L["conv"].shape != ((H + G) * D, m.taps):
+                                   torch.zeros(H + pad, dtype=dtype, device=dev)]).contiguous()
+            conv = torch.cat([F(p + "mix.q.conv"), F(p + "mix.k.conv")])
+            if conv.shape != ((H + G) * D, m.taps):
                 raise ValueError(f"layer {i}: convolution weights do not match the config")
+            L["conv"] = conv.t().contiguous()                 # tap-major [taps, C]
             L["q_norm"], L["k_norm"] = F(p + "mix.q.norm"), F(p + "mix.k.norm")
             L["pb"] = F(p + "mix.pb")
             L["wo"], L["bo"] = W(p + "mix.o"), W(p + "mix.o.b")
@@ -219,7 +224,8 @@ class SodonexModel:
             seqmix.seq_state_save(x, u, st["prev"], st["tail"], meta.state_slots, meta.cu_q,
                                   meta.positions)
             o = seqmix.sigmoid_attention(q, kc, vc, meta.cu_q, meta.ctx_lens, meta.block_tables,
-                                         meta.positions, L["pb"], u[:, (H + G) * D:], m.scale,
+                                         meta.positions, L["pb"],
+                                         u[:, (H + G) * D:(H + G) * D + H], m.scale,
                                          m.chunk, H, G, D, meta.max_q)
             y = ops.linear(o, L["wo"], L["bo"])
             f = lc.mlp

@@ -834,13 +834,13 @@ def conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm,
                           cos_sin, dims: int, H: int, G: int, D: int, k_cache, v_cache, slots,
                           out_dtype):
     """u [T, >= (H + G) D]: the projected q | k rows. Causal per-channel
-    convolution (weights conv_w [(H + G) D, taps], the rows before the feed from
+    convolution (weights conv_w tap-major [taps, (H + G) D], the rows before the feed from
     ``tail[slot]``), then: v = the convolved k; q and k each RMS-normed over the
     whole projection (weights q_norm / k_norm), rotated (rotate-half, the first
     ``dims`` entries of every head); k and v go to the paged caches
     [blocks, BLK, G D] at ``slots``; returns q [T, H D]."""
     T = u.shape[0]
-    C, taps = conv_w.shape
+    taps, C = conv_w.shape
     Cq = H * D
     cu = cu_q.tolist()
     y = torch.zeros(T, C, dtype=torch.float32, device=u.device)
@@ -857,7 +857,7 @@ def conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm,
             rows = u[q0:q1, :C].float()
         n = q1 - q0
         for j in range(taps):
-            y[q0:q1] += rows[j:j + n] * w[:, j]
+            y[q0:q1] += rows[j:j + n] * w[j]
     yq, yk = y[:, :Cq], y[:, Cq:]
     v = yk.to(v_cache.dtype)
     q = yq * torch.rsqrt(yq.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()

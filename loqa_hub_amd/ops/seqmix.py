@@ -426,8 +426,8 @@ def conv_norm_rope_append(u: torch.Tensor, conv_w: torch.Tensor, tail: torch.Ten
                           k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor,
                           out_dtype) -> torch.Tensor:
     """One launch between the q | k projection and attention: short causal
-    convolution per channel (f32 weights conv_w [(H + G) D, taps]; the rows
-    before a feed come from ``tail[slot]``), v = the convolved k, RMS norm of q
+    convolution per channel (f32 weights conv_w tap-major [taps, (H + G) D]; the
+    rows before a feed come from ``tail[slot]``), v = the convolved k, RMS norm of q
     and of k over the whole projection, rotate-half rotary on the first
     ``dims`` entries of every head, k and v into the paged caches
     [blocks, BLK, G D]; returns q [T, H D]."""
@@ -436,7 +436,7 @@ def conv_norm_rope_append(u: torch.Tensor, conv_w: torch.Tensor, tail: torch.Ten
                                          k_norm, eps, cos_sin, dims, H, G, D, k_cache, v_cache,
                                          slots, out_dtype)
     T = u.shape[0]
-    C, taps = conv_w.shape
+    taps, C = conv_w.shape
     assert C == (H + G) * D and u.stride(1) == 1 and u.shape[1] >= C
     _f32c(conv_w, "conv_w"); _f32c(tail, "tail"); _f32c(q_norm, "q_norm"); _f32c(k_norm, "k_norm")
     _f32c(cos_sin, "cos_sin"); _i32c(slots, "slots")

@@ -121,15 +121,16 @@ def test_token_shift_and_saved_row(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("extra", [3, 8], ids=["rows_unaligned", "rows_aligned"])
 @pytest.mark.parametrize("taps,dims", [(4, 8), (1, 16), (2, 0), (7, 4)])
-def test_conv_norm_rotary_append(device, taps, dims):
+def test_conv_norm_rotary_append(device, taps, dims, extra):
     """The launch between the projection and attention, fed in portions (some
     shorter than the convolution) into scattered page slots: q, the cached k
     and the cached v (= the convolved k before norm and rotation)."""
     g = torch.Generator().manual_seed(taps)
     H, G, D, n, eps, base = 3, 2, 16, 19, 1e-5, 100.0
     C = (H + G) * D
-    u = torch.randn(n, C + H, generator=g)                    # gate columns ride along
+    u = torch.randn(n, C + extra, generator=g)                # more columns ride along
     cw = torch.randn(C, taps, generator=g) * 0.5
     qn, kn = torch.rand(H * D, generator=g) + 0.5, torch.rand(G * D, generator=g) + 0.5
     y = O.short_conv(u[:, :C].double(), cw.double())
@@ -146,7 +147,7 @@ def test_conv_norm_rotary_append(device, taps, dims):
             cu, pos = _meta([c], [at], device)
             us = u[at:at + c].to(device)
             got.append(seqmix.conv_norm_rope_append(
-                us, cw.to(device), tail, slot, cu, pos, qn.to(device), kn.to(device), eps, table,
+                us, cw.t().contiguous().to(device), tail, slot, cu, pos, qn.to(device), kn.to(device), eps, table,
                 dims, H, G, D, kc, vc, where[at:at + c].to(device), torch.float32))
             seqmix.seq_state_save(None, us, None, tail, slot, cu, pos)
             at += c
