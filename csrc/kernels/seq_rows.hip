@@ -14,7 +14,8 @@
 // the q | k projection GEMM and attention: convolution in f32 (weights stored
 // tap-major, [taps][C]), v = convolved k, RMS norm over the whole q and the
 // whole k projection, rotate-half rotary positions on the first `dims` entries
-// of every head, k and v into their pages. The v8 form gives a thread 8
+// of every head, k into its page [blocks][BLK][G D] and v into its transposed
+// page [blocks][G D][BLK] (the layout attention reads). The v8 form gives a thread 8
 // neighbouring channels (16-byte loads and stores, all taps' loads in flight at
 // once); the scalar form takes any sizes.
 #include "seqmix.h"
@@ -78,7 +79,8 @@ __global__ __launch_bounds__(256) void conv_norm_rope_append_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ pos, int B,
     const float* __restrict__ qn, const float* __restrict__ kn, float eps,
     const float* __restrict__ cs, int max_pos, int dims, int H, int G, int D,
-    TO* __restrict__ kc, TO* __restrict__ vc, long cache_rows, const int* __restrict__ kvslots,
+    TO* __restrict__ kc, TO* __restrict__ vc, long cache_rows, int blk,
+    const int* __restrict__ kvslots,
     TO* __restrict__ q) {
   extern __shared__ float y[];                    // the convolved q | k row
   __shared__ float red[8];
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(256) void conv_norm_rope_append_kernel(
     if (isq) Act<TO>::st(q + (size_t)t * Cq + c, v);
     else if (store) {
       Act<TO>::st(kc + (size_t)slot * Ck + cc, v);
-      Act<TO>::st(vc + (size_t)slot * Ck + cc, y[c]);
+      Act<TO>::st(vc + ((size_t)(slot / blk) * Ck + cc) * blk + slot % blk, y[c]);
     }
   }
 }
@@ -158,7 +160,8 @@ __global__ __launch_bounds__(1024) void conv_norm_rope_append_v8_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ pos, int B,
     const float* __restrict__ qn, const float* __restrict__ kn, float eps,
     const float* __restrict__ cs, int max_pos, int dims, int H, int G, int D,
-    TO* __restrict__ kc, TO* __restrict__ vc, long cache_rows, const int* __restrict__ kvslots,
+    TO* __restrict__ kc, TO* __restrict__ vc, long cache_rows, int blk,
+    const int* __restrict__ kvslots,
     TO* __restrict__ q) {
   extern __shared__ float y[];
   __shared__ float red[16];
@@ -229,7 +232,9 @@ __global__ __launch_bounds__(1024) void conv_norm_rope_append_v8_kernel(
     if (isq) Row8<TO>::st(q + (size_t)t * Cq + c, v);
     else if (store) {
       Row8<TO>::st(kc + (size_t)slot * Ck + cc, v);
-      Row8<TO>::st(vc + (size_t)slot * Ck + cc, raw);
+      TO* vp = vc + ((size_t)(slot / blk) * Ck + cc) * blk + slot % blk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Act<TO>::st(vp + (size_t)e * blk, raw[e]);
     }
   }
 }
@@ -287,7 +292,8 @@ extern "C" int loqa_conv_norm_rope_append(
 #define ARGS(TU, TO)                                                                            \
   (const TU*)u, ldu, (const float*)cw, taps, (const float*)tail, nslots, (const int*)sslots,    \
       (const int*)cu_q, (const int*)pos, B, (const float*)qn, (const float*)kn, eps,            \
-      (const float*)cs, max_pos, dims, H, G, D, (TO*)kc, (TO*)vc, rows, (const int*)kvslots,    \
+      (const float*)cs, max_pos, dims, H, G, D, (TO*)kc, (TO*)vc, rows, blk,                   \
+      (const int*)kvslots,                                                                      \
       (TO*)q
 #define GO(TU, TO)                                                                              \
   do {                                                                                          \

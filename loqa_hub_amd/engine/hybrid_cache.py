@@ -4,8 +4,8 @@ Two kinds of per-sequence memory share one sequence table:
 
 * **pages**: per caching attention layer either one tensor [blocks, BLK,
   width] (latent attention: the normalised latent row and the rotated shared
-  key part of each token) or a key and a value tensor [blocks, BLK, heads x
-  size] (``kv``). The pages of all layers follow ONE block table per sequence,
+  key part of each token) or a key tensor [blocks, BLK, heads x size] and a
+  transposed value tensor [blocks, heads x size, BLK] (``kv``). The pages of all layers follow ONE block table per sequence,
   handed out by the same block pool the Llama KV cache uses (native
   ``BlockPool``);
 * **state slots**: one slot per live sequence (the last slot is the write
@@ -97,9 +97,11 @@ class HybridCache:
                        for li, width in spec["latent"].items()}
         self.state = {li: torch.zeros(max_seqs + 1, H, D, Dv, dtype=torch.float32, device=dev)
                       for li, (H, D, Dv) in spec["state"].items()}
-        # key / value pages of plain (uncompressed) attention layers
+        # key pages and transposed value pages of plain (uncompressed) attention
+        # layers: the value product sums over a page's keys, so its kernels want
+        # a column's keys side by side
         self.kv = {li: (torch.zeros(num_blocks, block_size, kw, dtype=dtype, device=dev),
-                        torch.zeros(num_blocks, block_size, vw, dtype=dtype, device=dev))
+                        torch.zeros(num_blocks, vw, block_size, dtype=dtype, device=dev))
                    for li, (kw, vw) in spec.get("kv", {}).items()}
         # named per-sequence rows
         self.rows = {li: {name: torch.zeros(max_seqs + 1, *shape, dtype=torch.float32, device=dev)

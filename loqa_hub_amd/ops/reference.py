@@ -837,8 +837,8 @@ def conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm,
     convolution (weights conv_w tap-major [taps, (H + G) D], the rows before the feed from
     ``tail[slot]``), then: v = the convolved k; q and k each RMS-normed over the
     whole projection (weights q_norm / k_norm), rotated (rotate-half, the first
-    ``dims`` entries of every head); k and v go to the paged caches
-    [blocks, BLK, G D] at ``slots``; returns q [T, H D]."""
+    ``dims`` entries of every head); k goes to its paged cache [blocks, BLK, G D]
+    and v to its transposed pages [blocks, G D, BLK] at ``slots``; returns q [T, H D]."""
     T = u.shape[0]
     taps, C = conv_w.shape
     Cq = H * D
@@ -878,13 +878,14 @@ def conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm,
     ok = sl >= 0
     blk = k_cache.shape[1]
     k_cache[(sl // blk)[ok], (sl % blk)[ok]] = k.to(k_cache.dtype)[ok]
-    v_cache[(sl // blk)[ok], (sl % blk)[ok]] = v[ok]
+    v_cache[(sl // blk)[ok], :, (sl % blk)[ok]] = v[ok]
     return q.to(out_dtype)
 
 
 def sigmoid_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positions, head_bias,
                       gate, scale: float, chunk: int, H: int, G: int, D: int, out_dtype):
-    """q [T, H D] against the paged caches [blocks, BLK, G D]: a query at
+    """q [T, H D] against the paged k cache [blocks, BLK, G D] and the
+    transposed v pages [blocks, G D, BLK]: a query at
     position p sees keys j <= p (with ``chunk`` > 0 only those of its own
     chunk, j // chunk == p // chunk); a visible key weighs
     sigmoid(q . k * scale + head_bias[h]), not normalised over keys; head h's
@@ -903,7 +904,7 @@ def sigmoid_attention(q, k_cache, v_cache, cu_q, ctx_lens, block_tables, positio
         idx = torch.arange(L, device=q.device)
         tab = block_tables[b].long()
         kk = k_cache[tab[idx // blk], idx % blk].float().view(L, G, D)
-        vv = v_cache[tab[idx // blk], idx % blk].float().view(L, G, D)
+        vv = v_cache[tab[idx // blk], :, idx % blk].float().view(L, G, D)
         qpos = positions[q0:q1].long()
         seen = idx[None, :] <= qpos[:, None]
         if chunk > 0:

@@ -429,8 +429,8 @@ def conv_norm_rope_append(u: torch.Tensor, conv_w: torch.Tensor, tail: torch.Ten
     convolution per channel (f32 weights conv_w tap-major [taps, (H + G) D]; the
     rows before a feed come from ``tail[slot]``), v = the convolved k, RMS norm of q
     and of k over the whole projection, rotate-half rotary on the first
-    ``dims`` entries of every head, k and v into the paged caches
-    [blocks, BLK, G D]; returns q [T, H D]."""
+    ``dims`` entries of every head, k into its paged cache [blocks, BLK, G D]
+    and v into its transposed pages [blocks, G D, BLK]; returns q [T, H D]."""
     if not u.is_cuda:
         return ref.conv_norm_rope_append(u, conv_w, tail, state_slots, cu_q, positions, q_norm,
                                          k_norm, eps, cos_sin, dims, H, G, D, k_cache, v_cache,
@@ -442,8 +442,9 @@ def conv_norm_rope_append(u: torch.Tensor, conv_w: torch.Tensor, tail: torch.Ten
     _f32c(cos_sin, "cos_sin"); _i32c(slots, "slots")
     assert tail.shape[1:] == (taps - 1, C) and q_norm.numel() == H * D and k_norm.numel() == G * D
     assert dims % 2 == 0 and dims <= D and (dims == 0 or cos_sin.shape[1] * 2 == dims)
-    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert k_cache.shape[2] == G * D and k_cache.dtype == v_cache.dtype == out_dtype
+    assert v_cache.shape == (k_cache.shape[0], G * D, k_cache.shape[1])
     assert slots.numel() >= T
     B = _seq_args(state_slots, cu_q, positions, T)
     q = torch.empty(T, H * D, dtype=out_dtype, device=u.device)
@@ -465,7 +466,8 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       positions: torch.Tensor, head_bias: torch.Tensor, gate: torch.Tensor | None,
                       scale: float, chunk: int, H: int, G: int, D: int, max_q: int = 0,
                       matrix_cores: bool | None = None) -> torch.Tensor:
-    """Attention without softmax over paged K/V [blocks, BLK, G D]: a query at
+    """Attention without softmax over paged K [blocks, BLK, G D] and transposed
+    V pages [blocks, G D, BLK]: a query at
     position p sees keys j <= p - with ``chunk`` > 0 only those of its own chunk
     (j // chunk == p // chunk, counted from the sequence's start) - and a
     visible key weighs sigmoid(q . k * scale + head_bias[h]) (f32, not
@@ -478,8 +480,9 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                      head_bias, gate, scale, chunk, H, G, D, q.dtype)
     T = q.shape[0]
     assert q.is_contiguous() and q.shape[1] == H * D and H % G == 0
-    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert k_cache.shape[2] == G * D and k_cache.dtype == v_cache.dtype == q.dtype
+    assert v_cache.shape == (k_cache.shape[0], G * D, k_cache.shape[1])
     _i32c(cu_q, "cu_q"); _i32c(ctx_lens, "ctx_lens"); _i32c(block_tables, "block_tables")
     _i32c(positions, "positions"); _f32c(head_bias, "head_bias")
     B = ctx_lens.numel()

@@ -138,7 +138,7 @@ def test_conv_norm_rotary_append(device, taps, dims, extra):
     wk = O.rotate_half((O.rms(y[:, H * D:], eps) * kn.double()).view(n, G, D), dims, base)
     table = seqmix.rope_table_half(dims, 64, base, device)
     for cuts in ([n], [1] * n, [2, 1, 9, 3, 4]):
-        kc, vc = torch.zeros(4, 8, G * D, device=device), torch.zeros(4, 8, G * D, device=device)
+        kc, vc = torch.zeros(4, 8, G * D, device=device), torch.zeros(4, G * D, 8, device=device)
         tail = torch.full((2, taps - 1, C), 7.0, device=device)
         slot = torch.tensor([1], dtype=torch.int32, device=device)
         where = torch.randperm(32, generator=g)[:n].to(torch.int32)
@@ -154,7 +154,8 @@ def test_conv_norm_rotary_append(device, taps, dims, extra):
         rows = where.long()
         assert (torch.cat(got).cpu().double() - wq.reshape(n, -1)).abs().max() < 2e-5, cuts
         assert (kc.view(32, -1)[rows].cpu().double() - wk.reshape(n, -1)).abs().max() < 2e-5
-        assert (vc.view(32, -1)[rows].cpu().double() - y[:, H * D:]).abs().max() < 2e-5
+        vrows = vc.transpose(1, 2).reshape(32, -1)[rows]           # value pages are [G D, BLK]
+        assert (vrows.cpu().double() - y[:, H * D:]).abs().max() < 2e-5
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -172,7 +173,7 @@ def test_sigmoid_attention_op(device, H, G, D, chunk):
     scale = D ** -0.5
     pb = torch.randn(H, generator=g)
     nblk = sum(-(-n // blk) for n in lens)
-    kc, vc = torch.zeros(nblk, blk, G * D), torch.zeros(nblk, blk, G * D)
+    kc, vc = torch.zeros(nblk, blk, G * D), torch.zeros(nblk, G * D, blk)
     order = torch.randperm(nblk, generator=g).tolist()
     bt = torch.zeros(3, 16, dtype=torch.int32)
     qs, want, gates = [], [], []
@@ -189,7 +190,7 @@ def test_sigmoid_attention_op(device, H, G, D, chunk):
             bt[b, i] = page
             m = min(blk, n - i * blk)
             kc[page, :m] = k[i * blk:i * blk + m].reshape(m, -1)
-            vc[page, :m] = v[i * blk:i * blk + m].reshape(m, -1)
+            vc[page, :, :m] = v[i * blk:i * blk + m].reshape(m, -1).T
         f = feeds[b]
         qs.append(q[n - f:].reshape(f, -1)); gates.append(gate[n - f:]); want.append(o[n - f:].reshape(f, -1))
     cu, pos = _meta(feeds, [n - f for n, f in zip(lens, feeds)], device)
@@ -534,7 +535,7 @@ def test_sigmoid_attention_matrix_cores(H, G, D, chunk):
     scale = D ** -0.5
     pb = torch.randn(H, generator=g) - 1.0
     nblk = sum(-(-n // blk) for n in lens)
-    kc, vc = torch.zeros(nblk, blk, G * D), torch.zeros(nblk, blk, G * D)
+    kc, vc = torch.zeros(nblk, blk, G * D), torch.zeros(nblk, G * D, blk)
     order = torch.randperm(nblk, generator=g).tolist()
     bt = torch.zeros(4, 16, dtype=torch.int32)
     qs, want, gates = [], [], []
@@ -551,7 +552,7 @@ def test_sigmoid_attention_matrix_cores(H, G, D, chunk):
             bt[b, i] = page
             m = min(blk, n - i * blk)
             kc[page, :m] = k[i * blk:i * blk + m].reshape(m, -1).float()
-            vc[page, :m] = v[i * blk:i * blk + m].reshape(m, -1).float()
+            vc[page, :, :m] = v[i * blk:i * blk + m].reshape(m, -1).float().T
         f = feeds[b]
         qs.append(q[n - f:].reshape(f, -1)); gates.append(gate[n - f:]); want.append(o[n - f:].reshape(f, -1))
     cu, pos = _meta(feeds, [n - f for n, f in zip(lens, feeds)], "cuda")
