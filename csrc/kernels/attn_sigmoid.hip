@@ -138,7 +138,8 @@ template <> struct Vec8<float> {
 // through shuffles (groups) and LDS (waves) in a fixed order. Which wave, lane
 // and step a key lands on depends only on its position in the sequence.
 template <typename T, int RH, int DC, int BK>
-__global__ __launch_bounds__(512) void sigmoid_attn_keys_kernel(SigAttnParams p, int heads_per_wg) {
+__global__ __launch_bounds__(RH <= 4 ? 1024 : 512) void sigmoid_attn_keys_kernel(
+    SigAttnParams p, int heads_per_wg) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, NW = blockDim.x >> 6;
   const int t = blockIdx.x, g = blockIdx.y;
@@ -473,10 +474,10 @@ extern "C" int loqa_sigmoid_attention(
   }
   if (D >= 8 && (D & (D - 1)) == 0 && pages_ok) {
     const int rep = H / G;
-    const int nw = D <= 128 ? 8 : 4;                       // waves: key tiles in flight
     int rh = rep < 8 ? rep : 8;
-    if (rh * D > 1024 && nw == 8) rh = 1024 / D;           // LDS: (1 + nw) RH D floats
     if (rh * D > 2048) rh = 2048 / D;
+    // waves = key windows in flight; LDS holds (1 + waves) RH D floats
+    const int nw = rh * D <= 512 && rh <= 4 ? 16 : rh * D <= 1024 ? 8 : 4;
     const int zs = (rep + rh - 1) / rh;
     const int hpw = (rep + zs - 1) / zs;
     const int RH = hpw <= 1 ? 1 : hpw == 2 ? 2 : hpw <= 4 ? 4 : 8;

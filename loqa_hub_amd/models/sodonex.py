@@ -11,9 +11,11 @@ row). The mixer is attention without softmax:
 * q and k projections with biases, each followed by a short causal
   convolution per channel, then one RMS norm over the whole projection, then
   rotate-half rotary positions on the first ``rot.dims`` entries of each head;
-* the values are the keys as they leave the convolution (no value projection);
+* no value projection: the value vectors are the convolved keys, taken before
+  their norm and rotation;
 * a query sees the earlier keys of its own chunk of ``mask.size`` positions;
-  a visible key weighs sigmoid(q . k * scale + bias_h), not normalised;
+  a visible key weighs sigmoid(q . k * scale + bias_h), and the weights are
+  used as they are, without dividing by their sum;
 * each head's output is multiplied by sigmoid of a per-head gate projection of
   the mixer's input before the output projection (with bias).
 
