@@ -159,8 +159,8 @@ def test_conv_norm_rotary_append(device, taps, dims, extra):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("H,G,D,chunk", [(4, 2, 16, 8), (3, 3, 8, 5), (8, 1, 64, 64), (2, 1, 24, 1),
-                                         (4, 4, 128, 40), (2, 2, 16, 0)])
+@pytest.mark.parametrize("H,G,D,chunk", [(4, 2, 16, 8), (3, 3, 8, 5), (6, 2, 64, 48), (2, 1, 24, 1),
+                                         (4, 4, 128, 40), (2, 2, 16, 0), (5, 1, 32, 64)])
 def test_sigmoid_attention_op(device, H, G, D, chunk):
     """The attention op on a batch of three unequal sequences (one decoding a
     single token at the first position of a chunk) against the oracle: keys
@@ -205,7 +205,7 @@ def test_sigmoid_attention_op(device, H, G, D, chunk):
 @pytest.mark.parametrize("device", DEVICES)
 def test_router_top_softmax(device):
     g = torch.Generator().manual_seed(0)
-    for E, top in [(12, 3), (5, 5), (7, 1), (130, 4)]:
+    for E, top in [(10, 3), (5, 5), (7, 1), (130, 4)]:
         h = torch.randn(33, 16, generator=g)
         sd = {"r.router": torch.randn(E, 16, generator=g), "r.router.b": torch.randn(E, generator=g)}
         idx, wt = O.route(h.double(), sd, "r.", {"router": {"experts": E, "top": top}})
@@ -239,7 +239,7 @@ def test_scalar_norm_residual_step(device):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("layer", [
     (O.attn(), None),
-    (O.attn(heads=8, kv_heads=1, dim=64, chunk=16, dims=32), None),      # matrix-core head size
+    (O.attn(heads=4, kv_heads=1, dim=64, chunk=16, dims=16), None),      # matrix-core head size
     (O.attn(heads=2, kv_heads=2, dim=8, taps=1, chunk=1, dims=8), None),  # every token alone
     (O.attn(heads=5, kv_heads=5, dim=12, taps=6, chunk=100, dims=2), None),   # one chunk holds all
     (O.attn(), O.moe_ff()),
@@ -431,6 +431,26 @@ def test_first_tokens_and_taps(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_odd_sizes(device, dtype):
+    """A width, vocabulary, head size and expert width that are no multiples of
+    8 (no 16-byte rows anywhere), three query heads per key/value head."""
+    cfg = O.make_config([(O.attn(heads=3, kv_heads=1, dim=10, taps=3, chunk=9, dims=6),
+                          O.moe_ff(experts=5, top=2, ff=13)),
+                         (O.attn(heads=6, kv_heads=2, dim=14, taps=2, chunk=4, dims=14), None)],
+                        width=50, vocab=77)
+    sd = O.make_weights(cfg, 8)
+    toks = tokens(45, 77, 3)
+    want = O.forward(cfg, sd, toks)
+    eng = engine(cfg, sd, device, dtype, max_tokens=64)
+    got = feed(eng, eng.open_sequence(), toks, [20, 1, 1, 6, 17])
+    if dtype == torch.float32:
+        assert rel_err(got, want) < TOL[dtype]
+    else:
+        assert rel_err(got, want, 0.5) < TOL[dtype]
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_long_decode(device):
     """150 single-token steps over many chunks and pages."""
     cfg = O.make_config([(O.attn(heads=2, kv_heads=1, dim=8, taps=4, chunk=7, dims=4), None),
@@ -524,7 +544,7 @@ def test_trace_replay_program(tmp_path, full_model):
 
 # ------------------------------------------- matrix-core paths (bf16, GPU only)
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,G,D,chunk", [(8, 1, 64, 64), (4, 2, 128, 48), (40, 2, 64, 20),
+@pytest.mark.parametrize("H,G,D,chunk", [(6, 1, 64, 48), (4, 2, 128, 64), (40, 2, 64, 20),
                                          (3, 3, 64, 0), (12, 1, 128, 1000)])
 def test_sigmoid_attention_matrix_cores(H, G, D, chunk):
     """The bf16 matrix-core form against the row form and the f64 oracle on a
